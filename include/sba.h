@@ -1,0 +1,161 @@
+/*
+ * sba.h -- C ABI of libsba.so: stick-breaking attention for AMD Instinct MI355X (gfx950).
+ *
+ * Plain C, no torch types.  Every pointer is a DEVICE pointer unless stated otherwise; the
+ * library never allocates, frees or synchronises: outputs and workspaces are owned by the
+ * caller and all work is enqueued on the HIP stream handed in (a `hipStream_t` passed as
+ * `void*`; NULL = the null stream).  Return value: 0 = ok, negative = SBA_E_* (bad argument,
+ * nothing launched), positive = a hipError_t raised by a launch.
+ *
+ * The entry points replace the host launchers of the upstream Python package
+ * (paths relative to the upstream repository root):
+ *
+ *   sba_varlen_fwd  <->  varlen_fwd / _compileable_forward
+ *                        stickbreaking_attention/sb_varlen/sb_varlen_fwd.py:413-522
+ *   sba_varlen_bwd  <->  varlen_bwd / _compileable_backward
+ *                        stickbreaking_attention/sb_varlen/sb_varlen_bwd.py:484-641
+ *   sba_attn_fwd    <->  _fwd / _compileable_fwd
+ *                        stickbreaking_attention/sb_attn/sb_fwd.py:139-253
+ *   sba_attn_bwd    <->  _bwd / _compileable_backward
+ *                        stickbreaking_attention/sb_attn/sb_bwd.py:163-297
+ *
+ * Upstream lets PyTorch allocate outputs, the saved per-row statistic and the lock/count
+ * workspaces and passes raw pointers plus explicit strides to the kernels; this ABI keeps
+ * that ownership model.  What differs is the private state carried from forward to
+ * backward: instead of one fp32 log-remainder per row (upstream `neg_log_acc`) the forward
+ * fills a per-(row, 64-key tile) carry table that both backward kernels consume, so the
+ * backward needs neither locks nor atomics.
+ */
+#ifndef SBA_H_
+#define SBA_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SBA_VERSION 100
+
+/* error codes (negative returns) */
+#define SBA_E_NULL      (-1)  /* a required pointer is NULL                         */
+#define SBA_E_HEAD_DIM  (-2)  /* head_dim not in {64, 128}                          */
+#define SBA_E_DTYPE     (-3)  /* dtype not SBA_BF16                                 */
+#define SBA_E_SHAPE     (-4)  /* negative / inconsistent sizes                      */
+#define SBA_E_STRIDE    (-5)  /* a row start is not 16-byte aligned (stride % 8)    */
+#define SBA_E_WORKSPACE (-6)  /* workspace or table too small                       */
+#define SBA_E_ARCH      (-7)  /* current device is not gfx950                       */
+
+/* element types */
+#define SBA_BF16 1
+
+/* flags */
+#define SBA_ATTEND_CURRENT 1u   /* a token may attend to itself (upstream attend_current) */
+#define SBA_CU_INT64       2u   /* cu_seqlens holds int64 (else int32)                    */
+#define SBA_FIXED_LENGTH   8u   /* the problem is the fixed-length op: `batch` documents of
+                                   `tokens` tokens each, cu_seqlens ignored (sba_attn_*)   */
+#define SBA_PRODUCT_SPACE  4u   /* carry the stick as a running product instead of a
+                                   running log2 sum (same results to ~1e-6, fewer
+                                   transcendentals); must match between fwd and bwd       */
+
+/* A strided view over [batch, heads, tokens, head_dim]; the last dimension is contiguous.
+ * Strides are in ELEMENTS.  For packed variable-length input batch == 1 and stride_b is
+ * ignored.  For per-row tensors (rem, grad_rem) the head_dim axis is absent. */
+typedef struct sba_view {
+  void*   ptr;
+  int64_t stride_b;
+  int64_t stride_h;
+  int64_t stride_t;
+} sba_view;
+
+/* Problem description shared by all four entry points. */
+typedef struct sba_problem {
+  int32_t  dtype;        /* SBA_BF16                                                     */
+  int32_t  head_dim;     /* 64 or 128                                                    */
+  int32_t  heads;        /* H                                                            */
+  int32_t  batch;        /* B for the fixed-length op, 1 for varlen                      */
+  int32_t  tokens;       /* T: tokens per batch entry (fixed) / total packed tokens      */
+  int32_t  n_docs;       /* varlen: number of entries in cu_seqlens; fixed: ignored      */
+  int32_t  max_doc_len;  /* upper bound on any document length (fixed: == tokens); sizes
+                            the carry tables: a longer document makes the scheduler flag
+                            SBA_STATUS_DOC_TOO_LONG and all kernels return early         */
+  uint32_t flags;        /* SBA_ATTEND_CURRENT | SBA_CU_INT64 | SBA_PRODUCT_SPACE | ...  */
+  float    inv_temp;     /* logit scale (upstream logit_scale / inv_temp)                */
+  const void* cu_seqlens;/* varlen: inclusive cumulative document ends, WITHOUT a leading
+                            zero (upstream strips it, sb_varlen/__init__.py:72-74)       */
+} sba_problem;
+
+/* ---- sizes ------------------------------------------------------------------------------ */
+
+/* Bytes of the schedule workspace (tile lists + status words) for this problem. */
+size_t sba_schedule_bytes(const sba_problem* p);
+
+/* Bytes of ONE carry table (fp32 [heads][ceil(max_doc_len/64)][batch*tokens]).  The forward
+ * fills `stick_table`; the backward additionally needs a `grad_table` of the same size. */
+size_t sba_table_bytes(const sba_problem* p);
+
+/* ---- schedule --------------------------------------------------------------------------- */
+
+/* Builds, on the device, the list of 128-row query tiles and 64-key KV tiles from
+ * cu_seqlens (documents sorted longest first, tiles of a document newest first) and validates
+ * cu_seqlens.  `schedule` must hold sba_schedule_bytes() bytes.  The first int32 of the
+ * workspace is a status word (0 = ok, else SBA_STATUS_*), readable by the caller after the
+ * stream has drained.  Has no upstream counterpart as a separate call: upstream derives the
+ * tile of a program from its grid index inside `_forward` (sb_varlen_fwd.py:281-296). */
+int sba_build_schedule(const sba_problem* p, void* schedule, void* stream);
+
+#define SBA_STATUS_OK            0
+#define SBA_STATUS_BAD_CU        1   /* cu_seqlens not monotone or beyond `tokens`          */
+#define SBA_STATUS_DOC_TOO_LONG  2   /* a document is longer than max_doc_len               */
+
+/* ---- forward ---------------------------------------------------------------------------- */
+
+/* o[b,h,t,:] and rem[b,h,t] for every token that belongs to a document; tokens outside any
+ * document are left untouched (the caller zero-fills).  `stick_table` may be NULL when no
+ * backward will follow. */
+int sba_varlen_fwd(const sba_problem* p, const void* schedule,
+                   const sba_view* q, const sba_view* k, const sba_view* v,
+                   const sba_view* o, const sba_view* rem,
+                   float* stick_table, void* stream);
+
+int sba_attn_fwd(const sba_problem* p, const void* schedule,
+                 const sba_view* q, const sba_view* k, const sba_view* v,
+                 const sba_view* o, const sba_view* rem,
+                 float* stick_table, void* stream);
+
+/* ---- backward --------------------------------------------------------------------------- */
+
+/* dq, dk, dv for every token of every document (others untouched).  `stick_table` is the
+ * table the forward filled for the same problem and inputs; `grad_table` is scratch of the
+ * same size.  grad_rem may have ptr == NULL (treated as zeros). */
+int sba_varlen_bwd(const sba_problem* p, const void* schedule,
+                   const sba_view* q, const sba_view* k, const sba_view* v,
+                   const sba_view* grad_o, const sba_view* grad_rem,
+                   const float* stick_table, float* grad_table,
+                   const sba_view* dq, const sba_view* dk, const sba_view* dv,
+                   void* stream);
+
+int sba_attn_bwd(const sba_problem* p, const void* schedule,
+                 const sba_view* q, const sba_view* k, const sba_view* v,
+                 const sba_view* grad_o, const sba_view* grad_rem,
+                 const float* stick_table, float* grad_table,
+                 const sba_view* dq, const sba_view* dk, const sba_view* dv,
+                 void* stream);
+
+/* ---- misc ------------------------------------------------------------------------------- */
+
+int         sba_version(void);
+const char* sba_error_string(int code);
+
+/* Duration in milliseconds of the most recent launch of each kernel on this thread's last
+ * call, measured with HIP events on the caller's stream when timing is switched on
+ * (sba_set_timing(1)); used by the benchmark to time the dominant kernel where it runs.
+ * which: 0 = forward, 1 = backward dq pass, 2 = backward dk/dv pass.  Synchronises. */
+void  sba_set_timing(int on);
+float sba_last_kernel_ms(int which);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SBA_H_ */

@@ -1,0 +1,256 @@
+// C ABI of libsba.so (declarations and the upstream functions each entry point replaces are
+// in include/sba.h).  Host code only validates, sizes and launches.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "sba.h"
+#include "sba_kernels.hpp"
+
+namespace {
+
+using namespace sba;
+
+thread_local int g_timing = 0;
+thread_local float g_ms[3] = {0.f, 0.f, 0.f};
+
+inline int cdiv_i(long long a, long long b) { return (int)((a + b - 1) / b); }
+
+struct Sizes {
+  int n_docs;        // documents the scheduler sees (fixed: batch)
+  long long rows;    // batch * tokens
+  int n_q_max, n_kv_max, n_tt;
+};
+
+int check_problem(const sba_problem* p, bool fixed, Sizes* sz) {
+  if (p == nullptr) return SBA_E_NULL;
+  if (p->dtype != SBA_BF16) return SBA_E_DTYPE;
+  if (p->head_dim != 64 && p->head_dim != 128) return SBA_E_HEAD_DIM;
+  if (p->heads <= 0 || p->tokens < 0 || p->batch <= 0 || p->max_doc_len < 0) return SBA_E_SHAPE;
+  if (fixed != ((p->flags & SBA_FIXED_LENGTH) != 0)) return SBA_E_SHAPE;
+  if (fixed) {
+    if (p->max_doc_len != p->tokens) return SBA_E_SHAPE;
+  } else {
+    if (p->batch != 1 || p->n_docs < 0) return SBA_E_SHAPE;
+    if (p->n_docs > 0 && p->cu_seqlens == nullptr) return SBA_E_NULL;
+  }
+  sz->n_docs = fixed ? p->batch : p->n_docs;
+  sz->rows = (long long)p->batch * p->tokens;
+  sz->n_q_max = (int)(sz->rows / BM) + sz->n_docs + 1;
+  sz->n_kv_max = (int)(sz->rows / BN) + sz->n_docs + 1;
+  sz->n_tt = cdiv_i(p->max_doc_len > 0 ? p->max_doc_len : 1, BN);
+  return 0;
+}
+
+size_t schedule_bytes(const Sizes& sz) {
+  size_t words = SCHED_HDR + 4 * ((size_t)sz.n_q_max + sz.n_kv_max) + 5 * (size_t)sz.n_docs + 2;
+  return (words * sizeof(int) + 255) & ~(size_t)255;
+}
+
+int check_view(const sba_view* v, bool need_ptr) {
+  if (v == nullptr) return SBA_E_NULL;
+  if (need_ptr && v->ptr == nullptr) return SBA_E_NULL;
+  return 0;
+}
+
+// 16-byte vector loads/stores need every row start aligned: strides multiple of 8 elements.
+int check_mat(const sba_view* v) {
+  int e = check_view(v, true);
+  if (e) return e;
+  if ((v->stride_b % 8) || (v->stride_h % 8) || (v->stride_t % 8) || ((uintptr_t)v->ptr % 16)) return SBA_E_STRIDE;
+  return 0;
+}
+
+View to_view(const sba_view* v) {
+  View r;
+  r.ptr = v ? (char*)v->ptr : nullptr;
+  r.sb = v ? v->stride_b : 0;
+  r.sh = v ? v->stride_h : 0;
+  r.st = v ? v->stride_t : 0;
+  return r;
+}
+
+int check_arch() {
+  static int cached = -1;   // immutable once set
+  if (cached >= 0) return cached ? 0 : SBA_E_ARCH;
+  int dev = 0;
+  hipDeviceProp_t prop;
+  if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return SBA_E_ARCH;
+  cached = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? 1 : 0;
+  return cached ? 0 : SBA_E_ARCH;
+}
+
+struct Timer {
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipStream_t s;
+  int which;
+  bool on;
+  Timer(int which_, hipStream_t s_) : s(s_), which(which_), on(g_timing != 0) {
+    if (on) {
+      on = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess;
+      if (on) (void)hipEventRecord(e0, s);
+    }
+  }
+  ~Timer() {
+    if (on) {
+      (void)hipEventRecord(e1, s);
+      (void)hipEventSynchronize(e1);
+      float ms = 0.f;
+      if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess) g_ms[which] = ms;
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+  }
+};
+
+int fill_common(const sba_problem* p, const Sizes& sz, const void* schedule, KArgs* a) {
+  if (schedule == nullptr) return SBA_E_NULL;
+  a->sched = reinterpret_cast<const int*>(schedule);
+  a->kv_list_off = SCHED_HDR + 4 * sz.n_q_max;
+  a->heads = p->heads;
+  a->tokens = p->tokens;
+  a->n_tt = sz.n_tt;
+  a->rows_total = sz.rows;
+  a->inv_temp = p->inv_temp;
+  a->c = p->inv_temp * 1.4426950408889634f;
+  return 0;
+}
+
+int forward(const sba_problem* p, bool fixed, const void* schedule, const sba_view* q, const sba_view* k,
+            const sba_view* v, const sba_view* o, const sba_view* rem, float* stick, void* stream) {
+  Sizes sz;
+  int e = check_problem(p, fixed, &sz);
+  if (e) return e;
+  if ((e = check_mat(q)) || (e = check_mat(k)) || (e = check_mat(v)) || (e = check_mat(o))) return e;
+  if ((e = check_view(rem, true))) return e;
+  if ((e = check_arch())) return e;
+  if (sz.rows == 0 || sz.n_docs == 0) return 0;
+  KArgs a;
+  std::memset(&a, 0, sizeof(a));
+  if ((e = fill_common(p, sz, schedule, &a))) return e;
+  a.q = to_view(q); a.k = to_view(k); a.v = to_view(v); a.o = to_view(o); a.rem = to_view(rem);
+  a.stick = stick;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  Timer tm(0, s);
+  return (int)launch_fwd(a, p->head_dim, (p->flags & SBA_ATTEND_CURRENT) != 0,
+                         (p->flags & SBA_PRODUCT_SPACE) != 0, sz.n_q_max, s);
+}
+
+int backward(const sba_problem* p, bool fixed, const void* schedule, const sba_view* q, const sba_view* k,
+             const sba_view* v, const sba_view* go, const sba_view* grem, const float* stick, float* gtab,
+             const sba_view* dq, const sba_view* dk, const sba_view* dv, void* stream) {
+  Sizes sz;
+  int e = check_problem(p, fixed, &sz);
+  if (e) return e;
+  if ((e = check_mat(q)) || (e = check_mat(k)) || (e = check_mat(v)) || (e = check_mat(go)) ||
+      (e = check_mat(dq)) || (e = check_mat(dk)) || (e = check_mat(dv)))
+    return e;
+  if (stick == nullptr || gtab == nullptr) return SBA_E_NULL;
+  if ((e = check_arch())) return e;
+  if (sz.rows == 0 || sz.n_docs == 0) return 0;
+  KArgs a;
+  std::memset(&a, 0, sizeof(a));
+  if ((e = fill_common(p, sz, schedule, &a))) return e;
+  a.q = to_view(q); a.k = to_view(k); a.v = to_view(v); a.go = to_view(go);
+  a.grem = to_view(grem);
+  a.dq = to_view(dq); a.dk = to_view(dk); a.dv = to_view(dv);
+  a.stick = const_cast<float*>(stick);
+  a.gtab = gtab;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const bool ac = (p->flags & SBA_ATTEND_CURRENT) != 0, prod = (p->flags & SBA_PRODUCT_SPACE) != 0;
+  hipError_t he;
+  {
+    Timer tm(1, s);
+    he = launch_bwd_dq(a, p->head_dim, ac, prod, sz.n_q_max, s);
+  }
+  if (he != hipSuccess) return (int)he;
+  {
+    Timer tm(2, s);
+    he = launch_bwd_dkdv(a, p->head_dim, ac, prod, sz.n_kv_max, s);
+  }
+  return (int)he;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sba_version(void) { return SBA_VERSION; }
+
+const char* sba_error_string(int code) {
+  switch (code) {
+    case 0: return "ok";
+    case SBA_E_NULL: return "a required pointer is NULL";
+    case SBA_E_HEAD_DIM: return "head_dim must be 64 or 128";
+    case SBA_E_DTYPE: return "unsupported element type (bf16 only)";
+    case SBA_E_SHAPE: return "negative or inconsistent sizes";
+    case SBA_E_STRIDE: return "pointer or stride breaks 16-byte row alignment";
+    case SBA_E_WORKSPACE: return "workspace too small";
+    case SBA_E_ARCH: return "current device is not gfx950 (MI355X)";
+    default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+  }
+}
+
+size_t sba_schedule_bytes(const sba_problem* p) {
+  Sizes sz;
+  const bool fixed = p != nullptr && (p->flags & SBA_FIXED_LENGTH) != 0;
+  if (check_problem(p, fixed, &sz)) return 0;
+  return schedule_bytes(sz);
+}
+
+size_t sba_table_bytes(const sba_problem* p) {
+  Sizes sz;
+  const bool fixed = p != nullptr && (p->flags & SBA_FIXED_LENGTH) != 0;
+  if (check_problem(p, fixed, &sz)) return 0;
+  return (size_t)p->heads * (size_t)sz.n_tt * (size_t)sz.rows * sizeof(float);
+}
+
+int sba_build_schedule(const sba_problem* p, void* schedule, void* stream) {
+  Sizes sz;
+  const bool fixed = p != nullptr && (p->flags & SBA_FIXED_LENGTH) != 0;
+  int e = check_problem(p, fixed, &sz);
+  if (e) return e;
+  if (schedule == nullptr) return SBA_E_NULL;
+  if ((e = check_arch())) return e;
+  SchedArgs a;
+  a.cu = fixed ? nullptr : p->cu_seqlens;
+  a.cu_is64 = (p->flags & SBA_CU_INT64) ? 1 : 0;
+  a.n_docs = sz.n_docs;
+  a.tokens = p->tokens;
+  a.max_doc_len = p->max_doc_len;
+  a.n_q_max = sz.n_q_max;
+  a.n_kv_max = sz.n_kv_max;
+  a.out = reinterpret_cast<int*>(schedule);
+  return (int)launch_schedule(a, reinterpret_cast<hipStream_t>(stream));
+}
+
+int sba_varlen_fwd(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
+                   const sba_view* v, const sba_view* o, const sba_view* rem, float* stick_table,
+                   void* stream) {
+  return forward(p, false, schedule, q, k, v, o, rem, stick_table, stream);
+}
+
+int sba_attn_fwd(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
+                 const sba_view* v, const sba_view* o, const sba_view* rem, float* stick_table,
+                 void* stream) {
+  return forward(p, true, schedule, q, k, v, o, rem, stick_table, stream);
+}
+
+int sba_varlen_bwd(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
+                   const sba_view* v, const sba_view* grad_o, const sba_view* grad_rem,
+                   const float* stick_table, float* grad_table, const sba_view* dq, const sba_view* dk,
+                   const sba_view* dv, void* stream) {
+  return backward(p, false, schedule, q, k, v, grad_o, grad_rem, stick_table, grad_table, dq, dk, dv, stream);
+}
+
+int sba_attn_bwd(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
+                 const sba_view* v, const sba_view* grad_o, const sba_view* grad_rem,
+                 const float* stick_table, float* grad_table, const sba_view* dq, const sba_view* dk,
+                 const sba_view* dv, void* stream) {
+  return backward(p, true, schedule, q, k, v, grad_o, grad_rem, stick_table, grad_table, dq, dk, dv, stream);
+}
+
+void sba_set_timing(int on) { g_timing = on; }
+float sba_last_kernel_ms(int which) { return (which >= 0 && which < 3) ? g_ms[which] : 0.f; }
+
+}  // extern "C"

@@ -1,0 +1,295 @@
+// Device-side building blocks shared by the forward and backward kernels (gfx950 only).
+//
+// Orientation used everywhere: the score tile is computed TRANSPOSED, S^T = K . Q^T, with the
+// 32x32x16 bf16 MFMA.  In the accumulator layout of that instruction a lane owns ONE query
+// (column n = lane % 32) and 16 of the 32 keys of the sub-block (rows 8*(i/4) + 4*h + i%4 for
+// register i, h = lane / 32); the lane with the other h owns the other 16 keys of the same
+// query.  The running sums / products of stick-breaking attention run along the key axis, so
+// they become in-register chains plus one exchange between the two half-waves
+// (v_permlane32_swap) -- no LDS, no DPP row scans.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sba {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
+
+constexpr int BM = 128;  // query rows per workgroup tile (4 waves x 32 rows)
+constexpr int BN = 64;   // keys per KV tile; also the granularity of the carry tables
+constexpr int NT = 256;  // threads per workgroup
+
+// Schedule workspace layout (int32 words).
+constexpr int SCHED_STATUS = 0;
+constexpr int SCHED_NQ = 1;      // number of query tiles
+constexpr int SCHED_NKV = 2;     // number of KV tiles
+constexpr int SCHED_MAXLEN = 3;  // longest document found
+constexpr int SCHED_HDR = 16;    // tile lists start here
+
+struct Tile {
+  int tok_start;  // first token of the document inside the packed token axis (0 for fixed-length)
+  int doc_len;
+  int idx;        // tile index inside the document
+  int batch;      // batch entry (0 for varlen)
+};
+
+struct View {
+  char* ptr;
+  int64_t sb, sh, st;  // element strides
+};
+
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// Round-to-nearest-even fp32 -> bf16 pairs (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ bf16x2 cvt2(float a, float b) {
+  f32x2 f = {a, b};
+  return __builtin_convertvector(f, bf16x2);
+}
+
+__device__ __forceinline__ bf16x8 pack8(const float* p) {
+  bf16x2 a = cvt2(p[0], p[1]), b = cvt2(p[2], p[3]), c = cvt2(p[4], p[5]), d = cvt2(p[6], p[7]);
+  bf16x8 r;
+  r[0] = a[0]; r[1] = a[1]; r[2] = b[0]; r[3] = b[1];
+  r[4] = c[0]; r[5] = c[1]; r[6] = d[0]; r[7] = d[1];
+  return r;
+}
+
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 r;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r[i] = (__bf16)0.0f;
+  return r;
+}
+
+// Both half-waves' values of `t`: lo = the value held by lane (n, h=0), hi = by lane (n, h=1).
+__device__ __forceinline__ void both_halves(float t, float& lo, float& hi) {
+  unsigned u = __builtin_bit_cast(unsigned, t);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  lo = __builtin_bit_cast(float, (unsigned)r[0]);
+  hi = __builtin_bit_cast(float, (unsigned)r[1]);
+}
+
+// LDS transpose read (ds_read_b64_tr_b16).  Inside each block of 16 lanes, lane r receives,
+// for j = 0..3, element (r % 4) of the four 16-bit values addressed by lane (4*j + r/4).
+// With lane i pointing at row (base + i/4), column (col0 + 4*(i%4)) of a row-major tile, lane
+// r ends up with rows base..base+3 of column col0 + r: four consecutive contraction indices
+// for the matrix column that lane owns in an MFMA operand.
+__device__ __forceinline__ s16x4 lds_tr4(const unsigned short* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
+}
+
+// MFMA operand (8 contraction slots per lane) gathered from a ROW-MAJOR LDS tile whose rows
+// are the contraction index.  `p0` / `p1` address rows 0..3 / 4..7 of the lane's 8-row group
+// as described for lds_tr4.
+__device__ __forceinline__ bf16x8 lds_tr8(const unsigned short* p0, const unsigned short* p1) {
+  s16x4 a = lds_tr4(p0), b = lds_tr4(p1);
+  s16x8 r = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+  return __builtin_bit_cast(bf16x8, r);
+}
+
+__device__ __forceinline__ bf16x8 lds_row8(const unsigned short* p) {
+  return *reinterpret_cast<const bf16x8*>(p);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Scans over the 32 keys of one sub-block for the query a lane pair owns.
+// v[i] belongs to key 8*(i/4) + 4*h + (i%4).
+// ---------------------------------------------------------------------------------------------
+
+// v[i] <- base + sum of v over keys >= key(i).  Returns the plain total over the 32 keys.
+__device__ __forceinline__ float suffix_sum32(float (&v)[16], int h, float base) {
+  float lo[4], hi[4], w[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    float t = (v[4 * g] + v[4 * g + 1]) + (v[4 * g + 2] + v[4 * g + 3]);
+    both_halves(t, lo[g], hi[g]);
+    w[g] = lo[g] + hi[g];
+  }
+  float z[4];
+  z[3] = base;
+  z[2] = z[3] + w[3];
+  z[1] = z[2] + w[2];
+  z[0] = z[1] + w[1];
+  const float total = (w[0] + w[1]) + (w[2] + w[3]);
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    // keys of the h=1 lane in group g come after those of the h=0 lane
+    const float off = z[g] + (h == 0 ? hi[g] : 0.0f);
+    v[4 * g + 3] += off;
+    v[4 * g + 2] += v[4 * g + 3];
+    v[4 * g + 1] += v[4 * g + 2];
+    v[4 * g + 0] += v[4 * g + 1];
+  }
+  return total;
+}
+
+// v[i] <- base + sum of v over keys <= key(i).  Returns the plain total over the 32 keys.
+__device__ __forceinline__ float prefix_sum32(float (&v)[16], int h, float base) {
+  float lo[4], hi[4], w[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    float t = (v[4 * g] + v[4 * g + 1]) + (v[4 * g + 2] + v[4 * g + 3]);
+    both_halves(t, lo[g], hi[g]);
+    w[g] = lo[g] + hi[g];
+  }
+  float z[4];
+  z[0] = base;
+  z[1] = z[0] + w[0];
+  z[2] = z[1] + w[1];
+  z[3] = z[2] + w[2];
+  const float total = (w[0] + w[1]) + (w[2] + w[3]);
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const float off = z[g] + (h == 1 ? lo[g] : 0.0f);
+    v[4 * g + 0] += off;
+    v[4 * g + 1] += v[4 * g + 0];
+    v[4 * g + 2] += v[4 * g + 1];
+    v[4 * g + 3] += v[4 * g + 2];
+  }
+  return total;
+}
+
+// ex[i] <- base * product of r over keys > key(i) (exclusive).  Returns base * product of all.
+__device__ __forceinline__ float suffix_prod32_excl(const float (&r)[16], float (&ex)[16], int h,
+                                                    float base) {
+  float lo[4], hi[4], w[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    float t = (r[4 * g] * r[4 * g + 1]) * (r[4 * g + 2] * r[4 * g + 3]);
+    both_halves(t, lo[g], hi[g]);
+    w[g] = lo[g] * hi[g];
+  }
+  float z[4];
+  z[3] = base;
+  z[2] = z[3] * w[3];
+  z[1] = z[2] * w[2];
+  z[0] = z[1] * w[1];
+  const float total = z[0] * w[0];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const float off = z[g] * (h == 0 ? hi[g] : 1.0f);
+    ex[4 * g + 3] = off;
+    ex[4 * g + 2] = ex[4 * g + 3] * r[4 * g + 3];
+    ex[4 * g + 1] = ex[4 * g + 2] * r[4 * g + 2];
+    ex[4 * g + 0] = ex[4 * g + 1] * r[4 * g + 1];
+  }
+  return total;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Stick-breaking weights of one 32-key sub-block for the lane's query.
+//
+//   x      raw q.k accumulators (S^T layout), c = inv_temp * log2(e)
+//   k0     document-local index of the sub-block's first key
+//   qrow   document-local index of the lane's query
+//   carry  stick left after all visible keys NEWER than this sub-block:
+//          LOG space: log2 of it (<= 0);  PRODUCT space: the value itself.  Updated in place.
+//   p      out: weights A[q, key(i)]
+//   beta   out (NEED_BETA): sigmoid(z), 0 where masked
+//
+// Restates compute_block of the upstream Triton kernel
+// (stickbreaking_attention/sb_varlen/sb_varlen_fwd.py:26-78): base-2 softplus
+// (sb_varlen/softplus.py:34-51), band mask with masked log(1-beta) forced to 0, reverse
+// inclusive running sum inside the block plus the carried total, exp2.  The running sum is
+// kept in fp32 registers instead of upstream's bf16 triangular matmul.
+// ---------------------------------------------------------------------------------------------
+template <bool AC, bool PROD, bool BAND, bool NEED_BETA>
+__device__ __forceinline__ void stick_weights(const f32x16& x, float c, int k0, int qrow, int h,
+                                              float& carry, float (&p)[16], float (&beta)[16]) {
+  bool vis[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int key = k0 + 8 * (i >> 2) + 4 * h + (i & 3);
+    vis[i] = BAND ? (AC ? key <= qrow : key < qrow) : true;
+  }
+  if constexpr (PROD) {
+    float r[16], b[16], ex[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float e = fast_exp2(c * x[i]);   // overflow -> inf -> r = 0, b = 1: still right
+      r[i] = fast_rcp(1.0f + e);             // 1 - beta
+      b[i] = 1.0f - r[i];
+      if (BAND && !vis[i]) { r[i] = 1.0f; b[i] = 0.0f; }
+    }
+    carry = suffix_prod32_excl(r, ex, h, carry);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      p[i] = b[i] * ex[i];
+      if (NEED_BETA) beta[i] = b[i];
+    }
+  } else {
+    float xs[16], sp[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      // clamping the logit at 126 (log2 units) keeps 2^x finite; sigmoid is 1 - 2^-126 there
+      xs[i] = fminf(c * x[i], 126.0f);
+      const float t = 1.0f + fast_exp2(xs[i]);
+      sp[i] = fast_log2(t);                  // base-2 softplus = -log2(1 - beta)
+      if (NEED_BETA) beta[i] = 1.0f - fast_rcp(t);
+      if (BAND && !vis[i]) { sp[i] = 0.0f; if (NEED_BETA) beta[i] = 0.0f; }
+    }
+    const float total = suffix_sum32(sp, h, -carry);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      p[i] = fast_exp2(xs[i] - sp[i]);
+      if (BAND && !vis[i]) p[i] = 0.0f;
+    }
+    carry -= total;
+  }
+}
+
+// Is the 32-key sub-block starting at k0 entirely invisible / entirely visible to the 32
+// queries starting at qw0?
+template <bool AC>
+__device__ __forceinline__ bool sub_skip(int k0, int qw0) {
+  return AC ? (k0 > qw0 + 31) : (k0 >= qw0 + 31);
+}
+template <bool AC>
+__device__ __forceinline__ bool sub_full(int k0, int qw0) {
+  return AC ? (k0 + 31 <= qw0) : (k0 + 31 < qw0);
+}
+
+// Cooperative load of `rows` x D bf16 from global (row stride `st` elements, rows >= limit are
+// zero-filled) into a row-major LDS tile with row stride LROW.  16 bytes per thread per step.
+template <int D, int ROWS, int LROW>
+__device__ __forceinline__ void load_rows_to_regs(const __bf16* base, int64_t st, int row0, int limit,
+                                                  uint4 (&reg)[ROWS * (D / 8) / NT]) {
+  constexpr int C8 = D / 8;
+#pragma unroll
+  for (int j = 0; j < ROWS * C8 / NT; ++j) {
+    const int cidx = threadIdx.x + NT * j;
+    const int row = cidx / C8, c8 = cidx % C8;
+    const int g = row0 + row;
+    if (g < limit) {
+      reg[j] = *reinterpret_cast<const uint4*>(base + (int64_t)g * st + c8 * 8);
+    } else {
+      reg[j] = make_uint4(0, 0, 0, 0);
+    }
+  }
+}
+
+template <int D, int ROWS, int LROW>
+__device__ __forceinline__ void store_regs_to_lds(unsigned short* lds,
+                                                  const uint4 (&reg)[ROWS * (D / 8) / NT]) {
+  constexpr int C8 = D / 8;
+#pragma unroll
+  for (int j = 0; j < ROWS * C8 / NT; ++j) {
+    const int cidx = threadIdx.x + NT * j;
+    const int row = cidx / C8, c8 = cidx % C8;
+    *reinterpret_cast<uint4*>(lds + row * LROW + c8 * 8) = reg[j];
+  }
+}
+
+}  // namespace sba

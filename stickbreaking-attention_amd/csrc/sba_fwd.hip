@@ -1,0 +1,146 @@
+// Forward kernel: one 128-row query tile of one (document, head) per workgroup, KV tiles of
+// 64 keys walked from the causal diagonal back to the start of the document.
+//
+// Replaces upstream `_forward` / `_forward_one_row`
+// (stickbreaking_attention/sb_varlen/sb_varlen_fwd.py:81-215, :231-410) and the fixed-length
+// wrapper (stickbreaking_attention/sb_attn/sb_fwd.py:15-136).
+#include "sba_kernels.hpp"
+
+namespace sba {
+
+template <int D, bool AC, bool PROD>
+__global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
+  constexpr int KS = D / 16;     // contraction steps of K.Q^T
+  constexpr int DB = D / 32;     // 32-wide output column blocks of P.V
+  constexpr int KROW = D + 8;    // K tile: row (b128) reads, stride = 4 banks mod 64
+  constexpr int VROW = D + 32;   // V tile: transpose reads, stride = 16 banks mod 64
+  constexpr int NCH = BN * (D / 8) / NT;
+  __shared__ __attribute__((aligned(16))) unsigned short Ks[BN * KROW];
+  __shared__ __attribute__((aligned(16))) unsigned short Vs[BN * VROW];
+
+  const int* sched = a.sched;
+  if (sched[SCHED_STATUS] != 0) return;
+  const int slot = blockIdx.x / a.heads;
+  const int head = blockIdx.x - slot * a.heads;
+  if (slot >= sched[SCHED_NQ]) return;
+  const Tile t = reinterpret_cast<const Tile*>(sched + SCHED_HDR)[slot];
+
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63, n = lane & 31, h = lane >> 5;
+  const int m0 = t.idx * BM;
+  const int qw0 = m0 + 32 * w;
+  const int qrow = qw0 + n;
+  const bool qvalid = qrow < t.doc_len;
+
+  const int64_t tok0 = t.tok_start;
+  const __bf16* qb = reinterpret_cast<const __bf16*>(a.q.ptr) + t.batch * a.q.sb + head * a.q.sh + tok0 * a.q.st;
+  const __bf16* kb = reinterpret_cast<const __bf16*>(a.k.ptr) + t.batch * a.k.sb + head * a.k.sh + tok0 * a.k.st;
+  const __bf16* vb = reinterpret_cast<const __bf16*>(a.v.ptr) + t.batch * a.v.sb + head * a.v.sh + tok0 * a.v.st;
+  __bf16* ob = reinterpret_cast<__bf16*>(a.o.ptr) + t.batch * a.o.sb + head * a.o.sh + tok0 * a.o.st;
+  __bf16* rb = reinterpret_cast<__bf16*>(a.rem.ptr) + t.batch * a.rem.sb + head * a.rem.sh + tok0 * a.rem.st;
+  const int64_t grow = (int64_t)t.batch * a.tokens + tok0 + qrow;  // row index in the tables
+
+  // Q^T operand fragments: lane (n, h) holds Q[qrow][16*ks + 8*h .. +7].
+  bf16x8 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    qf[ks] = qvalid ? *reinterpret_cast<const bf16x8*>(qb + (int64_t)qrow * a.q.st + 16 * ks + 8 * h)
+                    : zero8();
+  }
+
+  f32x16 oacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) oacc[db][i] = 0.0f;
+  float carry = PROD ? 1.0f : 0.0f;
+
+  const int last_key = min(m0 + BM - 1, t.doc_len - 1);
+  const int kt_last = last_key / BN;
+
+  // per-lane offset for the transpose reads of V: row 4*h + i/4, column 16*blk + 4*(i%4)
+  const int i16 = lane & 15, blk = (lane >> 4) & 1;
+  const int vtr = (4 * h + (i16 >> 2)) * VROW + 16 * blk + 4 * (i16 & 3);
+
+  uint4 kreg[NCH], vreg[NCH];
+  load_rows_to_regs<D, BN, KROW>(kb, a.k.st, kt_last * BN, t.doc_len, kreg);
+  load_rows_to_regs<D, BN, VROW>(vb, a.v.st, kt_last * BN, t.doc_len, vreg);
+
+  for (int kt = kt_last; kt >= 0; --kt) {
+    __syncthreads();
+    store_regs_to_lds<D, BN, KROW>(Ks, kreg);
+    store_regs_to_lds<D, BN, VROW>(Vs, vreg);
+    __syncthreads();
+    if (kt > 0) {
+      load_rows_to_regs<D, BN, KROW>(kb, a.k.st, (kt - 1) * BN, t.doc_len, kreg);
+      load_rows_to_regs<D, BN, VROW>(vb, a.v.st, (kt - 1) * BN, t.doc_len, vreg);
+    }
+    if (a.stick != nullptr && h == 0 && qvalid) {
+      a.stick[((int64_t)head * a.n_tt + kt) * a.rows_total + grow] = carry;
+    }
+#pragma unroll
+    for (int sb = 1; sb >= 0; --sb) {
+      const int k0 = kt * BN + 32 * sb;
+      if (sub_skip<AC>(k0, qw0)) continue;
+      f32x16 x;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) x[i] = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        x = mfma32(lds_row8(Ks + (32 * sb + n) * KROW + 16 * ks + 8 * h), qf[ks], x);
+      }
+      float p[16], unused[16];
+      if (sub_full<AC>(k0, qw0)) {
+        stick_weights<AC, PROD, false, false>(x, a.c, k0, qrow, h, carry, p, unused);
+      } else {
+        stick_weights<AC, PROD, true, false>(x, a.c, k0, qrow, h, carry, p, unused);
+      }
+      // P as the A operand of O = P.V: slot s of step tt is key 32*sb + 16*tt + 8*(s/4) + 4*h + s%4
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const bf16x8 pf = pack8(p + 8 * tt);
+        const unsigned short* vrow = Vs + vtr + (32 * sb + 16 * tt) * VROW;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const bf16x8 vf = lds_tr8(vrow + 32 * db, vrow + 8 * VROW + 32 * db);
+          oacc[db] = mfma32(pf, vf, oacc[db]);
+        }
+      }
+    }
+  }
+
+  // epilogue: rem = what is left of the stick; o rows in the accumulator layout
+  if (h == 0 && qvalid) {
+    const float r = PROD ? carry : fast_exp2(carry);
+    rb[(int64_t)qrow * a.rem.st] = (__bf16)r;
+  }
+#pragma unroll
+  for (int db = 0; db < DB; ++db) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = qw0 + 8 * (i >> 2) + 4 * h + (i & 3);
+      if (row < t.doc_len) ob[(int64_t)row * a.o.st + 32 * db + n] = (__bf16)oacc[db][i];
+    }
+  }
+}
+
+template <int D>
+static hipError_t launch_fwd_d(const KArgs& a, bool ac, bool prod, int n_q_max, hipStream_t s) {
+  const dim3 grid((unsigned)n_q_max * (unsigned)a.heads), block(NT);
+  if (ac) {
+    if (prod) hipLaunchKernelGGL((fwd_kernel<D, true, true>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((fwd_kernel<D, true, false>), grid, block, 0, s, a);
+  } else {
+    if (prod) hipLaunchKernelGGL((fwd_kernel<D, false, true>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((fwd_kernel<D, false, false>), grid, block, 0, s, a);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_fwd(const KArgs& a, int head_dim, bool ac, bool prod, int n_q_max, hipStream_t s) {
+  if (head_dim == 128) return launch_fwd_d<128>(a, ac, prod, n_q_max, s);
+  return launch_fwd_d<64>(a, ac, prod, n_q_max, s);
+}
+
+}  // namespace sba

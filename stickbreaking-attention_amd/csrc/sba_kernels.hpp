@@ -1,0 +1,43 @@
+// Kernel argument block and launch prototypes shared by the translation units of libsba.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "sba_device.hpp"
+
+namespace sba {
+
+struct KArgs {
+  View q, k, v, o, rem;        // forward tensors (rem has no head_dim axis)
+  View go, grem, dq, dk, dv;   // backward tensors (grem.ptr may be null)
+  const int* sched;            // schedule workspace
+  int kv_list_off;             // int32 offset of the KV tile list inside `sched`
+  float* stick;                // carry table written by the forward (may be null in fwd)
+  float* gtab;                 // gradient prefix table (backward scratch)
+  int heads;
+  int tokens;                  // tokens per batch entry
+  int n_tt;                    // table tiles per row = ceil(max_doc_len / BN)
+  int64_t rows_total;          // batch * tokens
+  float c;                     // inv_temp * log2(e)
+  float inv_temp;
+};
+
+struct SchedArgs {
+  const void* cu;   // null for fixed-length
+  int cu_is64;
+  int n_docs;       // documents (fixed: batch)
+  int tokens;       // T per batch entry
+  int max_doc_len;
+  int n_q_max, n_kv_max;
+  int* out;
+};
+
+hipError_t launch_schedule(const SchedArgs& a, hipStream_t s);
+hipError_t launch_fwd(const KArgs& a, int head_dim, bool attend_current, bool product, int n_q_max,
+                      hipStream_t s);
+hipError_t launch_bwd_dq(const KArgs& a, int head_dim, bool attend_current, bool product, int n_q_max,
+                         hipStream_t s);
+hipError_t launch_bwd_dkdv(const KArgs& a, int head_dim, bool attend_current, bool product,
+                           int n_kv_max, hipStream_t s);
+
+}  // namespace sba

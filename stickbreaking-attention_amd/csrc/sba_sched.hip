@@ -1,0 +1,152 @@
+// Device-side tile scheduler: turns cu_seqlens into the tile lists the compute kernels index
+// with blockIdx, without a device-to-host round trip.
+//
+// Upstream sizes its grid from the host-side `max_seqlens` and lets every program find its
+// document from cu_seqlens, pairing a long and a short causal row of two heads per program
+// (stickbreaking_attention/sb_varlen/sb_varlen_fwd.py:281-296, :476-480).  Here documents are
+// ranked longest first and each contributes exactly its own tiles, most expensive first, so
+// no program is idle and the tail of the launch is made of the cheapest tiles.
+#include "sba_kernels.hpp"
+
+namespace sba {
+
+constexpr int SCHED_THREADS = 1024;
+constexpr int RANK_LIMIT = 4096;   // beyond this many documents the input order is kept
+
+__device__ __forceinline__ int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// Scratch (int32) behind the two tile lists, per document: start, len, order, qoff, kvoff.
+__global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a) {
+  __shared__ int s_status, s_maxlen;
+  __shared__ int s_scan_q[SCHED_THREADS], s_scan_kv[SCHED_THREADS];
+  const int tid = threadIdx.x;
+  const int nd = a.n_docs;
+  int* hdr = a.out;
+  Tile* qtiles = reinterpret_cast<Tile*>(a.out + SCHED_HDR);
+  Tile* kvtiles = qtiles + a.n_q_max;
+  int* dstart = reinterpret_cast<int*>(kvtiles + a.n_kv_max);
+  int* dlen = dstart + nd;
+  int* order = dlen + nd;
+  int* qoff = order + nd;         // nd + 1 entries
+  int* kvoff = qoff + nd + 1;     // nd + 1 entries
+  const bool fixed = a.cu == nullptr;
+
+  if (tid == 0) { s_status = 0; s_maxlen = 0; }
+  __syncthreads();
+
+  // A. document bounds + validation
+  for (int d = tid; d < nd; d += SCHED_THREADS) {
+    long long st = 0, en = a.tokens;
+    if (!fixed) {
+      if (a.cu_is64) {
+        const long long* cu = reinterpret_cast<const long long*>(a.cu);
+        st = d ? cu[d - 1] : 0; en = cu[d];
+      } else {
+        const int* cu = reinterpret_cast<const int*>(a.cu);
+        st = d ? cu[d - 1] : 0; en = cu[d];
+      }
+    }
+    int len = 0;
+    if (st < 0 || en < st || en > a.tokens) {
+      atomicOr(&s_status, 1);   // SBA_STATUS_BAD_CU
+      st = 0;
+    } else {
+      len = (int)(en - st);
+      if (len > a.max_doc_len) atomicOr(&s_status, 2);   // SBA_STATUS_DOC_TOO_LONG
+    }
+    dstart[d] = (int)st;
+    dlen[d] = len;
+    atomicMax(&s_maxlen, len);
+  }
+  __syncthreads();
+
+  // B. rank documents by length, longest first (ties by index)
+  for (int d = tid; d < nd; d += SCHED_THREADS) {
+    int r = d;
+    if (!fixed && nd <= RANK_LIMIT) {
+      const int len = dlen[d];
+      r = 0;
+      for (int e = 0; e < nd; ++e) {
+        const int le = dlen[e];
+        r += (le > len) || (le == len && e < d);
+      }
+    }
+    order[r] = d;
+  }
+  __syncthreads();
+
+  // C. exclusive prefix of the tile counts in ranked order
+  const int per = cdiv(nd, SCHED_THREADS);
+  int sq = 0, skv = 0;
+  for (int j = 0; j < per; ++j) {
+    const int i = tid * per + j;
+    if (i < nd) {
+      const int len = dlen[order[i]];
+      sq += cdiv(len, BM);
+      skv += cdiv(len, BN);
+    }
+  }
+  s_scan_q[tid] = sq;
+  s_scan_kv[tid] = skv;
+  __syncthreads();
+  for (int off = 1; off < SCHED_THREADS; off <<= 1) {
+    int vq = 0, vkv = 0;
+    if (tid >= off) { vq = s_scan_q[tid - off]; vkv = s_scan_kv[tid - off]; }
+    __syncthreads();
+    s_scan_q[tid] += vq;
+    s_scan_kv[tid] += vkv;
+    __syncthreads();
+  }
+  int bq = s_scan_q[tid] - sq, bkv = s_scan_kv[tid] - skv;
+  for (int j = 0; j < per; ++j) {
+    const int i = tid * per + j;
+    if (i < nd) {
+      const int len = dlen[order[i]];
+      qoff[i] = bq; kvoff[i] = bkv;
+      bq += cdiv(len, BM);
+      bkv += cdiv(len, BN);
+    }
+  }
+  const int total_q = s_scan_q[SCHED_THREADS - 1], total_kv = s_scan_kv[SCHED_THREADS - 1];
+  if (tid == 0) { qoff[nd] = total_q; kvoff[nd] = total_kv; }
+  __syncthreads();
+
+  // D. emit tiles: slot -> ranked document by binary search over the prefix
+  const bool ok = s_status == 0;
+  for (int s = tid; s < total_q && ok; s += SCHED_THREADS) {
+    int lo = 0, hi = nd;   // largest i with qoff[i] <= s
+    while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (qoff[mid] <= s) lo = mid; else hi = mid; }
+    const int d = order[lo];
+    const int nq = cdiv(dlen[d], BM);
+    Tile t;
+    t.tok_start = fixed ? 0 : dstart[d];
+    t.doc_len = dlen[d];
+    t.idx = nq - 1 - (s - qoff[lo]);     // newest (most expensive) query tile first
+    t.batch = fixed ? d : 0;
+    qtiles[s] = t;
+  }
+  for (int s = tid; s < total_kv && ok; s += SCHED_THREADS) {
+    int lo = 0, hi = nd;
+    while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (kvoff[mid] <= s) lo = mid; else hi = mid; }
+    const int d = order[lo];
+    Tile t;
+    t.tok_start = fixed ? 0 : dstart[d];
+    t.doc_len = dlen[d];
+    t.idx = s - kvoff[lo];               // oldest keys are seen by the most queries: first
+    t.batch = fixed ? d : 0;
+    kvtiles[s] = t;
+  }
+  if (tid == 0) {
+    hdr[SCHED_STATUS] = s_status;
+    hdr[SCHED_NQ] = ok ? total_q : 0;
+    hdr[SCHED_NKV] = ok ? total_kv : 0;
+    hdr[SCHED_MAXLEN] = s_maxlen;
+  }
+}
+
+hipError_t launch_schedule(const SchedArgs& a, hipStream_t s) {
+  hipLaunchKernelGGL(sched_kernel, dim3(1), dim3(SCHED_THREADS), 0, s, a);
+  return hipGetLastError();
+}
+
+}  // namespace sba

@@ -1,0 +1,92 @@
+"""CPU-only checks of the boundary: the shared library loads, exports every symbol the header
+declares, sizes workspaces sensibly and rejects bad arguments without touching a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from stickbreaking_attention import _native as nat
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "sba.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sba_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = nat.load()
+    syms = header_symbols()
+    assert len(syms) >= 11
+    for s in syms:
+        assert hasattr(lib, s), f"{s} declared in include/sba.h but not exported"
+    assert sorted(nat.EXPORTS) == syms
+    assert lib.sba_version() == 100
+
+
+def problem(**kw):
+    base = dict(dtype=1, head_dim=128, heads=32, batch=1, tokens=16384, n_docs=8, max_doc_len=4096,
+                flags=0, inv_temp=0.0884, cu_seqlens=0x1000)
+    base.update(kw)
+    return nat.SbaProblem(*[base[f[0]] for f in nat.SbaProblem._fields_])
+
+
+def test_workspace_sizes():
+    lib = nat.load()
+    p = problem()
+    sched = lib.sba_schedule_bytes(ctypes.byref(p))
+    # two tile lists (16 B per tile) bounded by tokens/128 + docs and tokens/64 + docs
+    assert 16 * (128 + 8 + 256 + 8) <= sched <= 16 * (128 + 256 + 32) + 1024
+    assert lib.sba_table_bytes(ctypes.byref(p)) == 32 * 64 * 16384 * 4
+    pf = problem(batch=4, heads=16, tokens=2048, n_docs=0, max_doc_len=2048, head_dim=64,
+                 flags=nat.FLAG_FIXED_LENGTH, cu_seqlens=None)
+    assert lib.sba_table_bytes(ctypes.byref(pf)) == 16 * 32 * 4 * 2048 * 4
+
+
+@pytest.mark.parametrize("kw,code", [
+    (dict(head_dim=50), -2), (dict(dtype=7), -3), (dict(heads=0), -4), (dict(batch=2), -4),
+    (dict(cu_seqlens=None), -1),
+])
+def test_bad_problems_are_rejected_on_the_host(kw, code):
+    lib = nat.load()
+    p = problem(**kw)
+    assert lib.sba_schedule_bytes(ctypes.byref(p)) == 0
+    assert lib.sba_build_schedule(ctypes.byref(p), ctypes.c_void_p(0x1000), None) == code
+    v = nat.SbaView(0x1000, 0, 128 * 16384, 128)
+    r = nat.SbaView(0x1000, 0, 16384, 1)
+    assert lib.sba_varlen_fwd(ctypes.byref(p), ctypes.c_void_p(0x1000), ctypes.byref(v), ctypes.byref(v),
+                              ctypes.byref(v), ctypes.byref(v), ctypes.byref(r), None, None) == code
+
+
+def test_misaligned_stride_and_null_views_are_rejected():
+    lib = nat.load()
+    p = problem()
+    good = nat.SbaView(0x1000, 0, 128 * 16384, 128)
+    bad = nat.SbaView(0x1000, 0, 128 * 16384 + 2, 128)
+    null = nat.SbaView(None, 0, 0, 0)
+    r = nat.SbaView(0x1000, 0, 16384, 1)
+    args = lambda q: (ctypes.byref(p), ctypes.c_void_p(0x1000), ctypes.byref(q), ctypes.byref(good),
+                      ctypes.byref(good), ctypes.byref(good), ctypes.byref(r), None, None)
+    assert lib.sba_varlen_fwd(*args(bad)) == -5
+    assert lib.sba_varlen_fwd(*args(null)) == -1
+    assert b"16-byte" in lib.sba_error_string(-5)
+
+
+def test_ops_fail_loudly_without_a_gpu():
+    from stickbreaking_attention import sb_attn, sb_attn_varlen
+    q = torch.zeros(2, 16, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="MI355X"):
+        sb_attn_varlen(q, q, q, torch.tensor([16], dtype=torch.int32), 16, zero_start=False)
+    with pytest.raises(RuntimeError, match="MI355X"):
+        sb_attn(q[None], q[None], q[None])
+
+
+def test_missing_library_raises(monkeypatch):
+    monkeypatch.setattr(nat, "_lib", None)
+    monkeypatch.setattr(nat, "LIB_PATH", "/nonexistent/libsba.so")
+    with pytest.raises(RuntimeError, match="libsba.so not found"):
+        nat.load()

@@ -1,0 +1,309 @@
+"""GPU parity tests: the HIP path (through the Python operators, which call libsba.so through
+its C ABI) against the fp32 CPU oracle on identical bf16-rounded inputs, against the
+committed float64 fixtures, and -- at the benchmark's full sizes -- through properties that
+need no oracle.  Tolerance: max-abs 2e-2 on o, rem, dq, dk, dv (see helpers.assert_close for
+how bf16 output rounding of large values enters)."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import sb_oracle as orc
+from tests.helpers import (GOLDEN_DIR, assert_close, cu_from_lengths, doc_lengths, oracle_fixed,
+                           oracle_varlen)
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import ctypes
+    from stickbreaking_attention import _native as nat
+    assert os.path.exists(nat.LIB_PATH), "libsba.so must be built before the GPU tests run"
+    nat.load()
+
+
+def run_varlen(q, k, v, do, lengths, ac=False, drem=None, zero_start=False, cu_dtype=torch.int32,
+               inv_temp=None, max_seqlens="auto"):
+    from stickbreaking_attention import sb_attn_varlen
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    cu = cu_from_lengths(lengths, leading_zero=zero_start, dtype=cu_dtype, device=DEV)
+    ms = max(lengths) if max_seqlens == "auto" else max_seqlens
+    o, rem = sb_attn_varlen(qg, kg, vg, cu, ms, inv_temp=inv_temp, zero_start=zero_start, attend_current=ac)
+    outs, grads = (o,), (do.to(DEV),)
+    if drem is not None:
+        outs, grads = (o, rem), (do.to(DEV), drem.to(DEV))
+    dq, dk, dv = torch.autograd.grad(outs, (qg, kg, vg), grads)
+    torch.cuda.synchronize()
+    return o.detach(), rem.detach(), dq, dk, dv
+
+
+def check_all(got, ref, heads=None):
+    for name, g, r in zip(("o", "rem", "dq", "dk", "dv"), got, ref):
+        if heads is not None:
+            g = g[heads]
+        assert_close(name, g, r)
+
+
+# ---------------------------------------------------------------------------------------------
+# committed fixtures (float64 expectations)
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
+@pytest.mark.parametrize("product_space", [False, True])
+def test_golden_fixture(name, product_space, monkeypatch):
+    from stickbreaking_attention import _ops
+    monkeypatch.setattr(_ops, "PRODUCT_SPACE", product_space)
+    z = np.load(os.path.join(GOLDEN_DIR, "small_cases.npz"))
+    t = {k: torch.from_numpy(z[f"{name}_{k}"]) for k in ("q", "k", "v", "do", "dr", "o", "rem", "dq", "dk", "dv")}
+    lengths = [int(x) for x in z[f"{name}_lengths"]]
+    ac = bool(z[f"{name}_ac"][0])
+    bf = lambda x: x.to(torch.bfloat16)
+    got = run_varlen(bf(t["q"]), bf(t["k"]), bf(t["v"]), bf(t["do"]), lengths, ac, drem=bf(t["dr"]))
+    check_all(got, (t["o"], t["rem"], t["dq"], t["dk"], t["dv"]))
+
+
+# ---------------------------------------------------------------------------------------------
+# oracle comparisons on seeded inputs
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("product_space", [False, True])
+def test_config1_shape(product_space, monkeypatch):
+    """1 document x 512 tokens, 4 heads, d=64, N(0,1), strict causal."""
+    from stickbreaking_attention import _ops
+    monkeypatch.setattr(_ops, "PRODUCT_SPACE", product_space)
+    q, k, v, do = orc.make_inputs((4, 512, 64), 1337 + 1)
+    check_all(run_varlen(q, k, v, do, [512]), oracle_varlen(q, k, v, do, [512]))
+
+
+@pytest.mark.parametrize("lengths", [[1], [2], [3, 1, 1, 2], [63, 64, 65, 127, 128, 129, 1, 31, 33], [257, 640]])
+@pytest.mark.parametrize("ac", [False, True])
+@pytest.mark.parametrize("d", [64, 128])
+def test_ragged_documents(lengths, ac, d):
+    T = sum(lengths)
+    q, k, v, do = orc.make_inputs((3, T, d), 7 + T + d, dist="upstream")
+    g = torch.Generator().manual_seed(T)
+    drem = torch.randn((3, T), generator=g).to(torch.bfloat16)
+    check_all(run_varlen(q, k, v, do, lengths, ac, drem=drem), oracle_varlen(q, k, v, do, lengths, ac, drem=drem))
+
+
+def test_empty_documents_and_tail_tokens():
+    # zero-length documents in the middle, and 40 tokens after the last document
+    lengths = [50, 0, 0, 130, 0, 20]
+    T = sum(lengths) + 40
+    q, k, v, do = orc.make_inputs((2, T, 64), 11)
+    got = run_varlen(q, k, v, do, lengths)
+    ref = oracle_varlen(q, k, v, do, lengths)
+    check_all(got, ref)
+    for t in got:
+        assert (t[:, sum(lengths):] == 0).all(), "tokens outside every document must come back as zeros"
+
+
+@pytest.mark.parametrize("ac", [False, True])
+@pytest.mark.parametrize("H,L", [(3, 4096), (12, 4096), (3, 8192)])
+def test_upstream_varlen_grid(H, L, ac):
+    """The upstream test's own shapes and input distribution (single long document, d=128,
+    q shifted +1, k shifted -1, int64 cu_seqlens, o + rem*v epilogue in the caller)."""
+    from stickbreaking_attention import sb_attn_varlen
+    q, k, v, do = orc.make_inputs((H, L, 128), 1337, dist="upstream")
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    cu = cu_from_lengths([L], dtype=torch.int64, device=DEV)
+    o, rem = sb_attn_varlen(qg, kg, vg, cu_seqlens=cu, max_seqlens=L, inv_temp=1 / math.sqrt(128),
+                            zero_start=False, attend_current=ac)
+    out = o + rem[..., None] * vg
+    dq, dk, dv = torch.autograd.grad(out, (qg, kg, vg), do.to(DEV))
+    torch.cuda.synchronize()
+    qf, kf, vf = (t.float().requires_grad_() for t in (q, k, v))
+    ro, rrem = orc.sb_varlen(qf, kf, vf, [L], ac, row_chunk=1024)
+    rout = ro + rrem[..., None] * vf
+    rdq, rdk, rdv = torch.autograd.grad(rout, (qf, kf, vf), do.float())
+    assert_close("o+rem*v", out.detach(), rout.detach())
+    assert_close("dq", dq, rdq)
+    assert_close("dk", dk, rdk)
+    assert_close("dv", dv, rdv)
+
+
+@pytest.mark.parametrize("ac", [False, True])
+@pytest.mark.parametrize("B,H,T,d", [(2, 3, 500, 64), (1, 7, 256, 64), (2, 2, 1024, 128)])
+def test_fixed_length(B, H, T, d, ac):
+    from stickbreaking_attention import sb_attn
+    q, k, v, do = orc.make_inputs((B, H, T, d), 5 + T, dist="upstream")
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    o, rem = sb_attn(qg, kg, vg, attend_current=ac)
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do.to(DEV))
+    torch.cuda.synchronize()
+    check_all((o.detach(), rem.detach(), dq, dk, dv), oracle_fixed(q, k, v, do, ac))
+
+
+def test_config2_fixed_length_full():
+    """B=4, H=16, T=2048, d=64, N(0,1): kernel on the full problem, oracle per batch entry."""
+    from stickbreaking_attention import sb_attn
+    q, k, v, do = orc.make_inputs((4, 16, 2048, 64), 1337 + 2)
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    o, rem = sb_attn(qg, kg, vg)
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do.to(DEV))
+    torch.cuda.synchronize()
+    for b in range(4):
+        print(f" batch {b}")
+        ref = oracle_fixed(q[b:b + 1], k[b:b + 1], v[b:b + 1], do[b:b + 1])
+        check_all(tuple(t[b:b + 1] for t in (o.detach(), rem.detach(), dq, dk, dv)), ref)
+
+
+def test_config3_headline_varlen():
+    """32 heads, d=128, 16384 tokens in 8 documents: kernel on the full problem; the oracle
+    checks 4 of the 32 heads (all tokens) to stay within seconds."""
+    lengths = doc_lengths("c3")
+    q, k, v, do = orc.make_inputs((32, 16384, 128), 1337 + 3)
+    got = run_varlen(q, k, v, do, lengths)
+    heads = [0, 9, 22, 31]
+    ref = oracle_varlen(q[heads], k[heads], v[heads], do[heads], lengths, row_chunk=1024)
+    check_all(got, ref, heads=heads)
+
+
+def test_config4_many_short_documents():
+    """32 heads, d=64, 16384 tokens in ~200 documents of 16..256 tokens, zero_start=True."""
+    lengths = doc_lengths("c4")
+    q, k, v, do = orc.make_inputs((32, 16384, 64), 1337 + 4)
+    got = run_varlen(q, k, v, do, lengths, zero_start=True)
+    heads = list(range(0, 32, 4))
+    ref = oracle_varlen(q[heads], k[heads], v[heads], do[heads], lengths)
+    check_all(got, ref, heads=heads)
+
+
+def test_config5_long_context_forward():
+    """32 heads, d=128, 65536 tokens (one 32768-token document + 6 more), inputs x0.5, forward
+    only.  Oracle: heads 0 and 17, all rows, evaluated 1024 query rows at a time."""
+    from stickbreaking_attention import sb_attn_varlen
+    lengths = doc_lengths("c5")
+    q, k, v, _ = orc.make_inputs((32, 65536, 128), 1337 + 5, scale=0.5)
+    cu = cu_from_lengths(lengths, device=DEV)
+    with torch.no_grad():
+        o, rem = sb_attn_varlen(q.to(DEV), k.to(DEV), v.to(DEV), cu, max(lengths), zero_start=False)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all() and torch.isfinite(rem.float()).all()
+    heads = [0, 17]
+    with torch.no_grad():
+        ro, rrem = orc.sb_varlen(q[heads].float(), k[heads].float(), v[heads].float(), lengths, row_chunk=1024)
+    assert_close("o", o[heads], ro)
+    assert_close("rem", rem[heads], rrem)
+
+
+# ---------------------------------------------------------------------------------------------
+# properties at full size (no oracle)
+# ---------------------------------------------------------------------------------------------
+def test_full_size_properties_config3():
+    from stickbreaking_attention import sb_attn, sb_attn_varlen
+    lengths = doc_lengths("c3")
+    q, k, v, _ = orc.make_inputs((32, 16384, 128), 1337 + 3)
+    q, k, v = q.to(DEV), k.to(DEV), v.to(DEV)
+    cu = cu_from_lengths(lengths, device=DEV)
+    with torch.no_grad():
+        o, rem = sb_attn_varlen(q, k, v, cu, max(lengths), zero_start=False)
+        # (1) with v == 1 every output column is the stick that was used: o = 1 - rem
+        ones = torch.ones_like(v)
+        o1, rem1 = sb_attn_varlen(q, k, ones, cu, max(lengths), zero_start=False)
+        assert torch.equal(rem1, rem)
+        assert ((o1.float() - (1 - rem1.float())[..., None]).abs().max().item()) < 1e-2
+        assert (rem.float() >= 0).all() and (rem.float() <= 1).all()
+        # (2) first token of every document: o = 0, rem = 1
+        starts = [0] + list(np.cumsum(lengths)[:-1])
+        assert (o[:, starts] == 0).all() and (rem[:, starts] == 1).all()
+        # (3) document independence: the packed result equals each document run on its own
+        s = 0
+        for n in lengths[:3]:
+            od, remd = sb_attn(q[None, :, s:s + n], k[None, :, s:s + n], v[None, :, s:s + n])
+            assert torch.equal(od[0], o[:, s:s + n]) and torch.equal(remd[0], rem[:, s:s + n])
+            s += n
+        # (4) the op is linear in v
+        o2, _ = sb_attn_varlen(q, k, (2 * v), cu, max(lengths), zero_start=False)
+        assert ((o2.float() - 2 * o.float()).abs().max().item()) < 3e-2
+    torch.cuda.synchronize()
+
+
+def test_backward_is_deterministic():
+    lengths = [700, 300, 1100]
+    q, k, v, do = orc.make_inputs((4, sum(lengths), 128), 3)
+    a = run_varlen(q, k, v, do, lengths)
+    b = run_varlen(q, k, v, do, lengths)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+
+
+# ---------------------------------------------------------------------------------------------
+# API behaviour
+# ---------------------------------------------------------------------------------------------
+def test_zero_start_int64_and_inv_temp():
+    lengths = [100, 260, 77]
+    q, k, v, do = orc.make_inputs((2, sum(lengths), 64), 21)
+    got = run_varlen(q, k, v, do, lengths, zero_start=True, cu_dtype=torch.int64, inv_temp=0.2)
+    check_all(got, oracle_varlen(q, k, v, do, lengths, inv_temp=0.2))
+
+
+def test_token_major_layout_keeps_strides():
+    """Inputs stored [tokens, heads, d] and viewed as [heads, tokens, d] (how the upstream
+    benchmark feeds the op): o keeps q's strides, results unchanged."""
+    from stickbreaking_attention import sb_attn_varlen
+    lengths = [300, 212]
+    T, H, d = sum(lengths), 4, 128
+    q, k, v, do = orc.make_inputs((H, T, d), 5)
+    tm = lambda t: t.to(DEV).permute(1, 0, 2).contiguous().permute(1, 0, 2)
+    qg, kg, vg = (tm(t).requires_grad_() for t in (q, k, v))
+    assert qg.stride() == (d, H * d, 1)
+    o, rem = sb_attn_varlen(qg, kg, vg, cu_from_lengths(lengths, device=DEV), max(lengths), zero_start=False)
+    assert o.stride() == qg.stride() and o.dtype == torch.bfloat16 and rem.shape == (H, T)
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), tm(do))
+    torch.cuda.synchronize()
+    check_all((o.detach(), rem.detach(), dq, dk, dv), oracle_varlen(q, k, v, do, lengths))
+
+
+@pytest.mark.parametrize("d", [16, 32, 50, 96])
+def test_other_head_dims_run_zero_padded(d):
+    from stickbreaking_attention import sb_attn
+    q, k, v, do = orc.make_inputs((1, 2, 200, d), d, dist="upstream")
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    o, rem = sb_attn(qg, kg, vg)
+    assert o.shape == q.shape
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do.to(DEV))
+    torch.cuda.synchronize()
+    check_all((o.detach(), rem.detach(), dq, dk, dv), oracle_fixed(q, k, v, do))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_other_dtypes_are_computed_in_bf16(dtype):
+    from stickbreaking_attention import sb_attn
+    q, k, v, do = orc.make_inputs((1, 2, 160, 64), 9, dist="upstream")   # bf16-representable values
+    qg, kg, vg = (t.to(DEV).to(dtype).requires_grad_() for t in (q, k, v))
+    o, rem = sb_attn(qg, kg, vg)
+    assert o.dtype == dtype and rem.dtype == dtype
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do.to(DEV).to(dtype))
+    assert dq.dtype == dtype and dk.dtype == dtype
+    torch.cuda.synchronize()
+    check_all((o.detach(), rem.detach(), dq, dk, dv), oracle_fixed(q, k, v, do))
+
+
+def test_malformed_cu_seqlens_are_reported(monkeypatch):
+    from stickbreaking_attention import _ops, sb_attn_varlen
+    monkeypatch.setattr(_ops, "VALIDATE", True)
+    q = torch.zeros(2, 256, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError, match="non-decreasing"):
+        sb_attn_varlen(q, q, q, torch.tensor([100, 50, 256], dtype=torch.int32, device=DEV), 256, zero_start=False)
+    with pytest.raises(ValueError, match="non-decreasing"):
+        sb_attn_varlen(q, q, q, torch.tensor([100, 300], dtype=torch.int32, device=DEV), 256, zero_start=False)
+    with pytest.raises(ValueError, match="longer than max_seqlens"):
+        sb_attn_varlen(q, q, q, torch.tensor([200, 256], dtype=torch.int32, device=DEV), 64, zero_start=False)
+    with pytest.raises(AssertionError):
+        sb_attn_varlen(q, q, q, torch.tensor([5, 256], dtype=torch.int32, device=DEV), 256, zero_start=True)
+    torch.cuda.synchronize()
+
+
+def test_forward_only_needs_no_table():
+    from stickbreaking_attention import sb_attn_varlen
+    q, k, v, _ = orc.make_inputs((2, 300, 64), 2)
+    with torch.no_grad():
+        o, rem = sb_attn_varlen(q.to(DEV), k.to(DEV), v.to(DEV), cu_from_lengths([300], device=DEV), 300, zero_start=False)
+    ro, rrem = orc.sb_varlen(q.float(), k.float(), v.float(), [300])
+    assert_close("o", o, ro)
+    assert_close("rem", rem, rrem)
