@@ -148,8 +148,8 @@ int sba_attn_bwd(const sba_problem* p, const void* schedule,
 int         sba_version(void);
 const char* sba_error_string(int code);
 
-/* Duration in milliseconds of the most recent launch of each kernel on this thread's last
- * call, measured with HIP events on the caller's stream when timing is switched on
+/* Duration in milliseconds of the most recent launch of each kernel (process-wide: the
+ * backward may run on another thread), measured with HIP events on the caller's stream when timing is switched on
  * (sba_set_timing(1)); used by the benchmark to time the dominant kernel where it runs.
  * which: 0 = forward, 1 = backward dq pass, 2 = backward dk/dv pass.  Synchronises. */
 void  sba_set_timing(int on);

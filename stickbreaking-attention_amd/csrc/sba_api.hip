@@ -2,6 +2,7 @@
 // in include/sba.h).  Host code only validates, sizes and launches.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstring>
 
 #include "sba.h"
@@ -11,8 +12,9 @@ namespace {
 
 using namespace sba;
 
-thread_local int g_timing = 0;
-thread_local float g_ms[3] = {0.f, 0.f, 0.f};
+// Process-wide on purpose: PyTorch runs the backward on its own autograd thread.
+std::atomic<int> g_timing{0};
+std::atomic<float> g_ms[3];
 
 inline int cdiv_i(long long a, long long b) { return (int)((a + b - 1) / b); }
 
@@ -85,7 +87,7 @@ struct Timer {
   hipStream_t s;
   int which;
   bool on;
-  Timer(int which_, hipStream_t s_) : s(s_), which(which_), on(g_timing != 0) {
+  Timer(int which_, hipStream_t s_) : s(s_), which(which_), on(g_timing.load() != 0) {
     if (on) {
       on = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess;
       if (on) (void)hipEventRecord(e0, s);
@@ -96,7 +98,7 @@ struct Timer {
       (void)hipEventRecord(e1, s);
       (void)hipEventSynchronize(e1);
       float ms = 0.f;
-      if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess) g_ms[which] = ms;
+      if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess) g_ms[which].store(ms);
     }
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
@@ -250,7 +252,7 @@ int sba_attn_bwd(const sba_problem* p, const void* schedule, const sba_view* q, 
   return backward(p, true, schedule, q, k, v, grad_o, grad_rem, stick_table, grad_table, dq, dk, dv, stream);
 }
 
-void sba_set_timing(int on) { g_timing = on; }
-float sba_last_kernel_ms(int which) { return (which >= 0 && which < 3) ? g_ms[which] : 0.f; }
+void sba_set_timing(int on) { g_timing.store(on); }
+float sba_last_kernel_ms(int which) { return (which >= 0 && which < 3) ? g_ms[which].load() : 0.f; }
 
 }  // extern "C"
