@@ -23,7 +23,7 @@
  * workspaces and passes raw pointers plus explicit strides to the kernels; this ABI keeps
  * that ownership model.  What differs is the private state carried from forward to
  * backward: instead of one fp32 log-remainder per row (upstream `neg_log_acc`) the forward
- * fills a per-(row, 64-key tile) carry table that both backward kernels consume, so the
+ * fills a per-(row, 32-key block) carry table that both backward kernels consume, so the
  * backward needs neither locks nor atomics.
  */
 #ifndef SBA_H_
@@ -42,7 +42,8 @@ extern "C" {
 #define SBA_E_NULL      (-1)  /* a required pointer is NULL                         */
 #define SBA_E_HEAD_DIM  (-2)  /* head_dim not in {64, 128}                          */
 #define SBA_E_DTYPE     (-3)  /* dtype not SBA_BF16                                 */
-#define SBA_E_SHAPE     (-4)  /* negative / inconsistent sizes                      */
+#define SBA_E_SHAPE     (-4)  /* negative / inconsistent sizes, or tokens*stride_t
+                                 too large for 32-bit byte offsets (>= 2 GiB)       */
 #define SBA_E_STRIDE    (-5)  /* a row start is not 16-byte aligned (stride % 8)    */
 #define SBA_E_WORKSPACE (-6)  /* workspace or table too small                       */
 #define SBA_E_ARCH      (-7)  /* current device is not gfx950                       */
@@ -91,7 +92,7 @@ typedef struct sba_problem {
 /* Bytes of the schedule workspace (tile lists + status words) for this problem. */
 size_t sba_schedule_bytes(const sba_problem* p);
 
-/* Bytes of ONE carry table (fp32 [heads][ceil(max_doc_len/64)][batch*tokens]).  The forward
+/* Bytes of ONE carry table (fp32 [heads][ceil(max_doc_len/32)][batch*tokens]).  The forward
  * fills `stick_table`; the backward additionally needs a `grad_table` of the same size. */
 size_t sba_table_bytes(const sba_problem* p);
 

@@ -40,7 +40,7 @@ int check_problem(const sba_problem* p, bool fixed, Sizes* sz) {
   sz->rows = (long long)p->batch * p->tokens;
   sz->n_q_max = (int)(sz->rows / BM) + sz->n_docs + 1;
   sz->n_kv_max = (int)(sz->rows / BN) + sz->n_docs + 1;
-  sz->n_tt = cdiv_i(p->max_doc_len > 0 ? p->max_doc_len : 1, BN);
+  sz->n_tt = cdiv_i(p->max_doc_len > 0 ? p->max_doc_len : 1, BT);
   return 0;
 }
 
@@ -56,10 +56,14 @@ int check_view(const sba_view* v, bool need_ptr) {
 }
 
 // 16-byte vector loads/stores need every row start aligned: strides multiple of 8 elements.
-int check_mat(const sba_view* v) {
+// Tile loads address a (document, head) slice with 32-bit byte offsets: the token stride must
+// keep every row of the slice (plus one tile of slack) below 2 GiB.
+int check_mat(const sba_view* v, const sba_problem* p) {
   int e = check_view(v, true);
   if (e) return e;
   if ((v->stride_b % 8) || (v->stride_h % 8) || (v->stride_t % 8) || ((uintptr_t)v->ptr % 16)) return SBA_E_STRIDE;
+  if (v->stride_t < p->head_dim) return SBA_E_STRIDE;
+  if (((long long)p->tokens + 2 * BM) * v->stride_t * 2 >= (1ll << 31)) return SBA_E_SHAPE;
   return 0;
 }
 
@@ -123,7 +127,7 @@ int forward(const sba_problem* p, bool fixed, const void* schedule, const sba_vi
   Sizes sz;
   int e = check_problem(p, fixed, &sz);
   if (e) return e;
-  if ((e = check_mat(q)) || (e = check_mat(k)) || (e = check_mat(v)) || (e = check_mat(o))) return e;
+  if ((e = check_mat(q, p)) || (e = check_mat(k, p)) || (e = check_mat(v, p)) || (e = check_mat(o, p))) return e;
   if ((e = check_view(rem, true))) return e;
   if ((e = check_arch())) return e;
   if (sz.rows == 0 || sz.n_docs == 0) return 0;
@@ -144,8 +148,8 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, const sba_v
   Sizes sz;
   int e = check_problem(p, fixed, &sz);
   if (e) return e;
-  if ((e = check_mat(q)) || (e = check_mat(k)) || (e = check_mat(v)) || (e = check_mat(go)) ||
-      (e = check_mat(dq)) || (e = check_mat(dk)) || (e = check_mat(dv)))
+  if ((e = check_mat(q, p)) || (e = check_mat(k, p)) || (e = check_mat(v, p)) || (e = check_mat(go, p)) ||
+      (e = check_mat(dq, p)) || (e = check_mat(dk, p)) || (e = check_mat(dv, p)))
     return e;
   if (stick == nullptr || gtab == nullptr) return SBA_E_NULL;
   if ((e = check_arch())) return e;

@@ -2,9 +2,9 @@
 //
 // Orientation used everywhere: the score tile is computed TRANSPOSED, S^T = K . Q^T, with the
 // 32x32x16 bf16 MFMA.  In the accumulator layout of that instruction a lane owns ONE query
-// (column n = lane % 32) and 16 of the 32 keys of the sub-block (rows 8*(i/4) + 4*h + i%4 for
-// register i, h = lane / 32); the lane with the other h owns the other 16 keys of the same
-// query.  The running sums / products of stick-breaking attention run along the key axis, so
+// (column n = lane % 32) and 16 of the 32 rows of the sub-block (rows 8*(i/4) + 4*h + i%4 for
+// register i, h = lane / 32); the lane with the other h owns the other 16 rows of the same
+// query.  Which key sits in which row is ours to choose (see kperm).  The running sums / products of stick-breaking attention run along the key axis, so
 // they become in-register chains plus one exchange between the two half-waves
 // (v_permlane32_swap) -- no LDS, no DPP row scans.
 #pragma once
@@ -22,7 +22,8 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 
 constexpr int BM = 128;  // query rows per workgroup tile (4 waves x 32 rows)
-constexpr int BN = 64;   // keys per KV tile; also the granularity of the carry tables
+constexpr int BN = 64;   // keys per KV tile staged in LDS
+constexpr int BT = 32;   // keys per carry-table entry (one MFMA sub-block)
 constexpr int NT = 256;  // threads per workgroup
 
 // Schedule workspace layout (int32 words).
@@ -104,94 +105,56 @@ __device__ __forceinline__ bf16x8 lds_row8(const unsigned short* p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Scans over the 32 keys of one sub-block for the query a lane pair owns.
-// v[i] belongs to key 8*(i/4) + 4*h + (i%4).
+// Key ownership.  Row m of the S^T MFMA is fed with key  kperm(m) = 16*((m>>2)&1) + 4*(m>>3) + (m&3)
+// of the sub-block (the lane that supplies A-operand row m simply loads that key), so that in
+// the accumulator the lane with half-wave index h owns the 16 CONSECUTIVE keys 16*h + i
+// (register i).  Running sums / products along the keys are then one in-register chain plus a
+// single exchange between the half-waves.
 // ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ int kperm(int m) { return ((m & 4) << 2) | ((m >> 3) << 2) | (m & 3); }
+
+// ex[i] <- base * product of r over keys newer than key(i) (exclusive).  Returns base * all.
+__device__ __forceinline__ float suffix_prod32_excl(const float (&r)[16], float (&ex)[16], int h,
+                                                    float base) {
+  const float t = (((r[0] * r[1]) * (r[2] * r[3])) * ((r[4] * r[5]) * (r[6] * r[7]))) *
+                  (((r[8] * r[9]) * (r[10] * r[11])) * ((r[12] * r[13]) * (r[14] * r[15])));
+  float lo, hi;
+  both_halves(t, lo, hi);
+  // keys of the h=1 lane (16..31) are newer than those of the h=0 lane
+  ex[15] = h == 0 ? base * hi : base;
+#pragma unroll
+  for (int i = 14; i >= 0; --i) ex[i] = ex[i + 1] * r[i + 1];
+  return base * (lo * hi);
+}
 
 // v[i] <- base + sum of v over keys >= key(i).  Returns the plain total over the 32 keys.
 __device__ __forceinline__ float suffix_sum32(float (&v)[16], int h, float base) {
-  float lo[4], hi[4], w[4];
+  const float t = (((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]))) +
+                  (((v[8] + v[9]) + (v[10] + v[11])) + ((v[12] + v[13]) + (v[14] + v[15])));
+  float lo, hi;
+  both_halves(t, lo, hi);
+  v[15] += h == 0 ? base + hi : base;
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    float t = (v[4 * g] + v[4 * g + 1]) + (v[4 * g + 2] + v[4 * g + 3]);
-    both_halves(t, lo[g], hi[g]);
-    w[g] = lo[g] + hi[g];
-  }
-  float z[4];
-  z[3] = base;
-  z[2] = z[3] + w[3];
-  z[1] = z[2] + w[2];
-  z[0] = z[1] + w[1];
-  const float total = (w[0] + w[1]) + (w[2] + w[3]);
-#pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    // keys of the h=1 lane in group g come after those of the h=0 lane
-    const float off = z[g] + (h == 0 ? hi[g] : 0.0f);
-    v[4 * g + 3] += off;
-    v[4 * g + 2] += v[4 * g + 3];
-    v[4 * g + 1] += v[4 * g + 2];
-    v[4 * g + 0] += v[4 * g + 1];
-  }
-  return total;
+  for (int i = 14; i >= 0; --i) v[i] += v[i + 1];
+  return lo + hi;
 }
 
 // v[i] <- base + sum of v over keys <= key(i).  Returns the plain total over the 32 keys.
 __device__ __forceinline__ float prefix_sum32(float (&v)[16], int h, float base) {
-  float lo[4], hi[4], w[4];
+  const float t = (((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]))) +
+                  (((v[8] + v[9]) + (v[10] + v[11])) + ((v[12] + v[13]) + (v[14] + v[15])));
+  float lo, hi;
+  both_halves(t, lo, hi);
+  v[0] += h == 1 ? base + lo : base;
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    float t = (v[4 * g] + v[4 * g + 1]) + (v[4 * g + 2] + v[4 * g + 3]);
-    both_halves(t, lo[g], hi[g]);
-    w[g] = lo[g] + hi[g];
-  }
-  float z[4];
-  z[0] = base;
-  z[1] = z[0] + w[0];
-  z[2] = z[1] + w[1];
-  z[3] = z[2] + w[2];
-  const float total = (w[0] + w[1]) + (w[2] + w[3]);
-#pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const float off = z[g] + (h == 1 ? lo[g] : 0.0f);
-    v[4 * g + 0] += off;
-    v[4 * g + 1] += v[4 * g + 0];
-    v[4 * g + 2] += v[4 * g + 1];
-    v[4 * g + 3] += v[4 * g + 2];
-  }
-  return total;
-}
-
-// ex[i] <- base * product of r over keys > key(i) (exclusive).  Returns base * product of all.
-__device__ __forceinline__ float suffix_prod32_excl(const float (&r)[16], float (&ex)[16], int h,
-                                                    float base) {
-  float lo[4], hi[4], w[4];
-#pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    float t = (r[4 * g] * r[4 * g + 1]) * (r[4 * g + 2] * r[4 * g + 3]);
-    both_halves(t, lo[g], hi[g]);
-    w[g] = lo[g] * hi[g];
-  }
-  float z[4];
-  z[3] = base;
-  z[2] = z[3] * w[3];
-  z[1] = z[2] * w[2];
-  z[0] = z[1] * w[1];
-  const float total = z[0] * w[0];
-#pragma unroll
-  for (int g = 0; g < 4; ++g) {
-    const float off = z[g] * (h == 0 ? hi[g] : 1.0f);
-    ex[4 * g + 3] = off;
-    ex[4 * g + 2] = ex[4 * g + 3] * r[4 * g + 3];
-    ex[4 * g + 1] = ex[4 * g + 2] * r[4 * g + 2];
-    ex[4 * g + 0] = ex[4 * g + 1] * r[4 * g + 1];
-  }
-  return total;
+  for (int i = 1; i < 16; ++i) v[i] += v[i - 1];
+  return lo + hi;
 }
 
 // ---------------------------------------------------------------------------------------------
 // Stick-breaking weights of one 32-key sub-block for the lane's query.
 //
-//   x      raw q.k accumulators (S^T layout), c = inv_temp * log2(e)
+//   x      raw q.k accumulators (S^T layout, register i = key 16*h + i), c = inv_temp * log2(e)
 //   k0     document-local index of the sub-block's first key
 //   qrow   document-local index of the lane's query
 //   carry  stick left after all visible keys NEWER than this sub-block:
@@ -208,12 +171,8 @@ __device__ __forceinline__ float suffix_prod32_excl(const float (&r)[16], float 
 template <bool AC, bool PROD, bool BAND, bool NEED_BETA>
 __device__ __forceinline__ void stick_weights(const f32x16& x, float c, int k0, int qrow, int h,
                                               float& carry, float (&p)[16], float (&beta)[16]) {
-  bool vis[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int key = k0 + 8 * (i >> 2) + 4 * h + (i & 3);
-    vis[i] = BAND ? (AC ? key <= qrow : key < qrow) : true;
-  }
+  // visible keys of a band sub-block: key < qrow (<= with attend_current)  <=>  i < lim
+  const int lim = qrow - k0 - 16 * h + (AC ? 1 : 0);
   if constexpr (PROD) {
     float r[16], b[16], ex[16];
 #pragma unroll
@@ -221,7 +180,7 @@ __device__ __forceinline__ void stick_weights(const f32x16& x, float c, int k0, 
       const float e = fast_exp2(c * x[i]);   // overflow -> inf -> r = 0, b = 1: still right
       r[i] = fast_rcp(1.0f + e);             // 1 - beta
       b[i] = 1.0f - r[i];
-      if (BAND && !vis[i]) { r[i] = 1.0f; b[i] = 0.0f; }
+      if (BAND && !(i < lim)) { r[i] = 1.0f; b[i] = 0.0f; }
     }
     carry = suffix_prod32_excl(r, ex, h, carry);
 #pragma unroll
@@ -238,13 +197,13 @@ __device__ __forceinline__ void stick_weights(const f32x16& x, float c, int k0, 
       const float t = 1.0f + fast_exp2(xs[i]);
       sp[i] = fast_log2(t);                  // base-2 softplus = -log2(1 - beta)
       if (NEED_BETA) beta[i] = 1.0f - fast_rcp(t);
-      if (BAND && !vis[i]) { sp[i] = 0.0f; if (NEED_BETA) beta[i] = 0.0f; }
+      if (BAND && !(i < lim)) { sp[i] = 0.0f; if (NEED_BETA) beta[i] = 0.0f; }
     }
     const float total = suffix_sum32(sp, h, -carry);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       p[i] = fast_exp2(xs[i] - sp[i]);
-      if (BAND && !vis[i]) p[i] = 0.0f;
+      if (BAND && !(i < lim)) p[i] = 0.0f;
     }
     carry -= total;
   }
@@ -261,34 +220,83 @@ __device__ __forceinline__ bool sub_full(int k0, int qw0) {
   return AC ? (k0 + 31 <= qw0) : (k0 + 31 < qw0);
 }
 
-// Cooperative load of `rows` x D bf16 from global (row stride `st` elements, rows >= limit are
-// zero-filled) into a row-major LDS tile with row stride LROW.  16 bytes per thread per step.
-template <int D, int ROWS, int LROW>
-__device__ __forceinline__ void load_rows_to_regs(const __bf16* base, int64_t st, int row0, int limit,
-                                                  uint4 (&reg)[ROWS * (D / 8) / NT]) {
+// ---------------------------------------------------------------------------------------------
+// Global -> register tile loads through a buffer resource that covers exactly the rows of one
+// (document, head) slice: rows at or past the end of the document fall outside the resource
+// and the hardware returns zeros for them, so no branch and no 64-bit address arithmetic.
+// ---------------------------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+
+struct Rows {
+  __amdgpu_buffer_rsrc_t rsrc;
+  unsigned row_bytes;   // stride between consecutive tokens, in bytes
+};
+
+__device__ __forceinline__ Rows make_rows(const __bf16* base, int64_t stride_t, int n_rows) {
+  Rows r;
+  const uint64_t bytes = (uint64_t)n_rows * (uint64_t)stride_t * 2u;
+  r.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<__bf16*>(base), 0,
+                                             bytes > 0xffffffffull ? 0xffffffffu : (unsigned)bytes, 0x00020000);
+  r.row_bytes = (unsigned)stride_t * 2u;
+  return r;
+}
+
+__device__ __forceinline__ uint4 load16(const Rows& r, int row, int col_bytes) {
+  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r.rsrc, row * (int)r.row_bytes + col_bytes, 0, 0);
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+
+__device__ __forceinline__ bf16x8 load_frag(const Rows& r, int row, int col_bytes) {
+  return __builtin_bit_cast(bf16x8, load16(r, row, col_bytes));
+}
+
+// Cooperative load of ROWS x D bf16 (16 bytes per thread per step) by THREADS threads.
+// KEYS = true: the tile holds keys and register slot (m, chunk) receives key kperm(m) of its
+// 32-key sub-block, so that LDS row m is MFMA row m.
+template <int D, int ROWS, int THREADS, bool KEYS>
+__device__ __forceinline__ void load_tile(const Rows& r, int row0, uint4 (&reg)[ROWS * (D / 8) / THREADS]) {
   constexpr int C8 = D / 8;
 #pragma unroll
-  for (int j = 0; j < ROWS * C8 / NT; ++j) {
-    const int cidx = threadIdx.x + NT * j;
-    const int row = cidx / C8, c8 = cidx % C8;
-    const int g = row0 + row;
-    if (g < limit) {
-      reg[j] = *reinterpret_cast<const uint4*>(base + (int64_t)g * st + c8 * 8);
-    } else {
-      reg[j] = make_uint4(0, 0, 0, 0);
-    }
+  for (int j = 0; j < ROWS * C8 / THREADS; ++j) {
+    const int cidx = threadIdx.x + THREADS * j;
+    const int m = cidx / C8;
+    const int src = KEYS ? ((m & ~31) | kperm(m & 31)) : m;
+    reg[j] = load16(r, row0 + src, (cidx % C8) * 16);
   }
 }
 
-template <int D, int ROWS, int LROW>
-__device__ __forceinline__ void store_regs_to_lds(unsigned short* lds,
-                                                  const uint4 (&reg)[ROWS * (D / 8) / NT]) {
+// Store such a tile row-major into LDS with a padded row stride of LROW elements.
+template <int D, int ROWS, int THREADS, int LROW>
+__device__ __forceinline__ void store_tile_padded(unsigned short* lds, const uint4 (&reg)[ROWS * (D / 8) / THREADS]) {
   constexpr int C8 = D / 8;
 #pragma unroll
-  for (int j = 0; j < ROWS * C8 / NT; ++j) {
-    const int cidx = threadIdx.x + NT * j;
-    const int row = cidx / C8, c8 = cidx % C8;
-    *reinterpret_cast<uint4*>(lds + row * LROW + c8 * 8) = reg[j];
+  for (int j = 0; j < ROWS * C8 / THREADS; ++j) {
+    const int cidx = threadIdx.x + THREADS * j;
+    *reinterpret_cast<uint4*>(lds + (cidx / C8) * LROW + (cidx % C8) * 8) = reg[j];
+  }
+}
+
+// XOR swizzle of the 16-byte chunks of an UNPADDED row-major tile (row = D*2 bytes) that makes
+// both access patterns of a dual-use tile bank-conflict free: row reads (16 consecutive rows,
+// one chunk each) and transpose reads (4 consecutive rows, 64 contiguous bytes each).
+template <int D>
+__device__ __forceinline__ int swz(int row) {
+  if constexpr (D == 128) return ((row & 3) << 2) | ((row >> 2) & 3);
+  else { const int x = (row >> 1) & 7; return ((x & 1) << 2) | (x >> 1); }
+}
+
+template <int D>
+__device__ __forceinline__ int swz_off(int row, int chunk) {   // element offset of a 16-byte chunk
+  return row * D + ((chunk ^ swz<D>(row)) << 3);
+}
+
+template <int D, int ROWS, int THREADS>
+__device__ __forceinline__ void store_tile_swizzled(unsigned short* lds, const uint4 (&reg)[ROWS * (D / 8) / THREADS]) {
+  constexpr int C8 = D / 8;
+#pragma unroll
+  for (int j = 0; j < ROWS * C8 / THREADS; ++j) {
+    const int cidx = threadIdx.x + THREADS * j;
+    *reinterpret_cast<uint4*>(lds + swz_off<D>(cidx / C8, cidx % C8)) = reg[j];
   }
 }
 

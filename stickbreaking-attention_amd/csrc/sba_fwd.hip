@@ -40,14 +40,14 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
   __bf16* ob = reinterpret_cast<__bf16*>(a.o.ptr) + t.batch * a.o.sb + head * a.o.sh + tok0 * a.o.st;
   __bf16* rb = reinterpret_cast<__bf16*>(a.rem.ptr) + t.batch * a.rem.sb + head * a.rem.sh + tok0 * a.rem.st;
   const int64_t grow = (int64_t)t.batch * a.tokens + tok0 + qrow;  // row index in the tables
+  const Rows qrows = make_rows(qb, a.q.st, t.doc_len);
+  const Rows krows = make_rows(kb, a.k.st, t.doc_len);
+  const Rows vrows = make_rows(vb, a.v.st, t.doc_len);
 
-  // Q^T operand fragments: lane (n, h) holds Q[qrow][16*ks + 8*h .. +7].
+  // Q^T operand fragments: lane (n, h) holds Q[qrow][16*ks + 8*h .. +7] (zeros past the document).
   bf16x8 qf[KS];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    qf[ks] = qvalid ? *reinterpret_cast<const bf16x8*>(qb + (int64_t)qrow * a.q.st + 16 * ks + 8 * h)
-                    : zero8();
-  }
+  for (int ks = 0; ks < KS; ++ks) qf[ks] = load_frag(qrows, qrow, 32 * ks + 16 * h);
 
   f32x16 oacc[DB];
 #pragma unroll
@@ -62,27 +62,27 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
   // per-lane offset for the transpose reads of V: row 4*h + i/4, column 16*blk + 4*(i%4)
   const int i16 = lane & 15, blk = (lane >> 4) & 1;
   const int vtr = (4 * h + (i16 >> 2)) * VROW + 16 * blk + 4 * (i16 & 3);
+  float* stick = a.stick == nullptr ? nullptr : a.stick + (int64_t)head * a.n_tt * a.rows_total + grow;
 
   uint4 kreg[NCH], vreg[NCH];
-  load_rows_to_regs<D, BN, KROW>(kb, a.k.st, kt_last * BN, t.doc_len, kreg);
-  load_rows_to_regs<D, BN, VROW>(vb, a.v.st, kt_last * BN, t.doc_len, vreg);
+  load_tile<D, BN, NT, true>(krows, kt_last * BN, kreg);
+  load_tile<D, BN, NT, true>(vrows, kt_last * BN, vreg);
 
   for (int kt = kt_last; kt >= 0; --kt) {
     __syncthreads();
-    store_regs_to_lds<D, BN, KROW>(Ks, kreg);
-    store_regs_to_lds<D, BN, VROW>(Vs, vreg);
+    store_tile_padded<D, BN, NT, KROW>(Ks, kreg);
+    store_tile_padded<D, BN, NT, VROW>(Vs, vreg);
     __syncthreads();
     if (kt > 0) {
-      load_rows_to_regs<D, BN, KROW>(kb, a.k.st, (kt - 1) * BN, t.doc_len, kreg);
-      load_rows_to_regs<D, BN, VROW>(vb, a.v.st, (kt - 1) * BN, t.doc_len, vreg);
-    }
-    if (a.stick != nullptr && h == 0 && qvalid) {
-      a.stick[((int64_t)head * a.n_tt + kt) * a.rows_total + grow] = carry;
+      load_tile<D, BN, NT, true>(krows, (kt - 1) * BN, kreg);
+      load_tile<D, BN, NT, true>(vrows, (kt - 1) * BN, vreg);
     }
 #pragma unroll
     for (int sb = 1; sb >= 0; --sb) {
       const int k0 = kt * BN + 32 * sb;
       if (sub_skip<AC>(k0, qw0)) continue;
+      // stick left on entering this sub-block: what both backward kernels start it from
+      if (stick != nullptr && h == 0 && qvalid) stick[(int64_t)(2 * kt + sb) * a.rows_total] = carry;
       f32x16 x;
 #pragma unroll
       for (int i = 0; i < 16; ++i) x[i] = 0.0f;
@@ -96,7 +96,8 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
       } else {
         stick_weights<AC, PROD, true, false>(x, a.c, k0, qrow, h, carry, p, unused);
       }
-      // P as the A operand of O = P.V: slot s of step tt is key 32*sb + 16*tt + 8*(s/4) + 4*h + s%4
+      // P as the A operand of O = P.V: slot s of step tt is key 16*h + 8*tt + s, which the
+      // permuted tile keeps in LDS row 16*tt + 8*(s/4) + 4*h + s%4.
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt) {
         const bf16x8 pf = pack8(p + 8 * tt);

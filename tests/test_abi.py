@@ -41,10 +41,10 @@ def test_workspace_sizes():
     sched = lib.sba_schedule_bytes(ctypes.byref(p))
     # two tile lists (16 B per tile) bounded by tokens/128 + docs and tokens/64 + docs
     assert 16 * (128 + 8 + 256 + 8) <= sched <= 16 * (128 + 256 + 32) + 1024
-    assert lib.sba_table_bytes(ctypes.byref(p)) == 32 * 64 * 16384 * 4
+    assert lib.sba_table_bytes(ctypes.byref(p)) == 32 * 128 * 16384 * 4
     pf = problem(batch=4, heads=16, tokens=2048, n_docs=0, max_doc_len=2048, head_dim=64,
                  flags=nat.FLAG_FIXED_LENGTH, cu_seqlens=None)
-    assert lib.sba_table_bytes(ctypes.byref(pf)) == 16 * 32 * 4 * 2048 * 4
+    assert lib.sba_table_bytes(ctypes.byref(pf)) == 16 * 64 * 4 * 2048 * 4
 
 
 @pytest.mark.parametrize("kw,code", [
