@@ -63,7 +63,7 @@ int check_mat(const sba_view* v, const sba_problem* p) {
   if (e) return e;
   if ((v->stride_b % 8) || (v->stride_h % 8) || (v->stride_t % 8) || ((uintptr_t)v->ptr % 16)) return SBA_E_STRIDE;
   if (v->stride_t < p->head_dim) return SBA_E_STRIDE;
-  if (((long long)p->tokens + 2 * BM) * v->stride_t * 2 >= (1ll << 31)) return SBA_E_SHAPE;
+  if (((long long)p->tokens + 8 * BM) * v->stride_t * 2 >= (1ll << 31)) return SBA_E_SHAPE;
   return 0;
 }
 

@@ -23,24 +23,24 @@
 
 namespace sba {
 
-// One 32-key sub-block for the 32 queries of a wave, given the raw score and do.v^T
-// accumulators: p, beta from the stick carry at the sub-block's newer edge, G, then dz with
-// the running prefix of G (carry_c: in = prefix before the sub-block, out = after it).
-// Emits p and dz as bf16 A-operand fragments: slot s of fragment [tt] is key 16*h + 8*tt + s.
-template <bool AC, bool PROD, bool NEED_P>
-__device__ __forceinline__ void grad_block(const f32x16& x, const f32x16& da, float c, int k0, int qw0,
-                                           int qrow, int h, float carry_e, float& carry_c, float dr,
-                                           bf16x8 (&pf)[2], bf16x8 (&zf)[2]) {
-  float p[16], bt[16];
+// One 32-key sub-block for the 32 queries of a wave, in two phases so that the do.v^T
+// accumulators need not be live while the weights are formed:
+//   grad_weights  p, beta from the raw scores and the stick carry at the sub-block's newer edge
+//   grad_dz       G = p (do.v - drem), dz = G - beta C with the running prefix C of G
+//                 (carry_c: in = prefix before the sub-block, out = after it)
+// p and dz leave as bf16 A-operand fragments: slot s of fragment [tt] is key 16*h + 8*tt + s.
+template <bool AC, bool PROD>
+__device__ __forceinline__ void grad_weights(const f32x16& x, float c, int k0, int qw0, int qrow, int h,
+                                             float carry_e, float (&p)[16], float (&bt)[16]) {
   if (sub_full<AC>(k0, qw0)) {
     stick_weights<AC, PROD, false, true>(x, c, k0, qrow, h, carry_e, p, bt);
   } else {
     stick_weights<AC, PROD, true, true>(x, c, k0, qrow, h, carry_e, p, bt);
   }
-  if (NEED_P) {
-    pf[0] = pack8(p);
-    pf[1] = pack8(p + 8);
-  }
+}
+
+__device__ __forceinline__ void grad_dz(const float (&p)[16], const float (&bt)[16], const f32x16& da, int h,
+                                        float& carry_c, float dr, bf16x8 (&zf)[2]) {
   float g[16], cs[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) { g[i] = p[i] * (da[i] - dr); cs[i] = g[i]; }
@@ -124,11 +124,19 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   load_tile<D, BN, NT, true>(vrows, 0, vreg);
 
   for (int kt = 0; kt <= kt_last; ++kt) {
-    __syncthreads();
+    lds_barrier();
     store_tile_padded<D, BN, NT, KROW>(Ks, kreg);
     store_tile_padded<D, BN, NT, TROW>(Kt, kreg);
     store_tile_padded<D, BN, NT, KROW>(Vs, vreg);
-    __syncthreads();
+    lds_barrier();
+    // Table reads go out BEFORE the tile prefetch: loads retire in order, so a table value
+    // requested after the prefetch could only be consumed once the whole prefetch had landed.
+    float ce[2];
+#pragma unroll
+    for (int sb = 0; sb < 2; ++sb) {
+      ce[sb] = PROD ? 1.0f : 0.0f;
+      if (qvalid && !sub_skip<AC>(kt * BN + 32 * sb, qw0)) ce[sb] = stick[(int64_t)(2 * kt + sb) * a.rows_total];
+    }
     if (kt < kt_last) {
       load_tile<D, BN, NT, true>(krows, (kt + 1) * BN, kreg);
       load_tile<D, BN, NT, true>(vrows, (kt + 1) * BN, vreg);
@@ -138,21 +146,28 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
       const int k0 = kt * BN + 32 * sb;
       if (sub_skip<AC>(k0, qw0)) continue;
       const int64_t tix = (int64_t)(2 * kt + sb) * a.rows_total;
-      float carry_e = PROD ? 1.0f : 0.0f;
-      if (qvalid) {
-        carry_e = stick[tix];
-        if (h == 0) gtab[tix] = carry_c;
-      }
-      f32x16 x, da;
+      float carry_e = ce[sb];
+      if (qvalid && h == 0) gtab[tix] = carry_c;
+      float p[16], bt[16];
+      {
+        f32x16 x;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) { x[i] = 0.0f; da[i] = 0.0f; }
+        for (int i = 0; i < 16; ++i) x[i] = 0.0f;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        x = mfma32(lds_row8(Ks + (32 * sb + n) * KROW + 16 * ks + 8 * h), qf[ks], x);
-        da = mfma32(lds_row8(Vs + (32 * sb + n) * KROW + 16 * ks + 8 * h), dof[ks], da);
+        for (int ks = 0; ks < KS; ++ks)
+          x = mfma32(lds_row8(Ks + (32 * sb + n) * KROW + 16 * ks + 8 * h), qf[ks], x);
+        grad_weights<AC, PROD>(x, a.c, k0, qw0, qrow, h, carry_e, p, bt);
       }
-      bf16x8 pf[2], zf[2];
-      grad_block<AC, PROD, false>(x, da, a.c, k0, qw0, qrow, h, carry_e, carry_c, dr, pf, zf);
+      bf16x8 zf[2];
+      {
+        f32x16 da;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) da[i] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          da = mfma32(lds_row8(Vs + (32 * sb + n) * KROW + 16 * ks + 8 * h), dof[ks], da);
+        grad_dz(p, bt, da, h, carry_c, dr, zf);
+      }
       // dq += dz . K  (K as the B operand: transpose reads along keys)
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt) {
@@ -177,23 +192,52 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
 }
 
 // -------------------------------------------------------------------------------------------
-// dk / dv pass: 8 waves; wave (qg, sb) scores the 32 queries of group qg against the 32 keys
-// of sub-block sb (K and V fragments stay in registers for the whole kernel), stages p and dz
-// through LDS, then every wave accumulates two 32x32 blocks of dk or dv over all 128 queries.
+// dk / dv pass.  One workgroup owns 64 keys of one (document, head) and walks the queries that
+// can see them, 64 at a time.  Its 8 waves are specialised so that every SIMD hosts one
+// VALU-bound and one MFMA-bound wave that run concurrently:
+//
+//   waves 0-3  "score" waves (query group qg, key sub-block sb): recompute the 32x32 block of
+//              p and dz of step i (K and V fragments live in registers) and stage them in LDS.
+//              Software-pipelined: the two MFMA chains (q.k and do.v) of block i+1 are issued
+//              while the VALU works on block i.
+//   waves 4-7  "product" waves: accumulate dv = p^T dO and dk = dz^T Q of step i-1 from the
+//              staged blocks (each owns 32 keys x D of one of the two outputs), and do all the
+//              global -> LDS staging of the Q/dO tiles, two steps ahead.
+//
+// p/dz staging is double-buffered and the Q/dO tiles sit in a ring of four slots (in step i:
+// slot i-1 feeds the products, slot i+1 the score chains, slot i+2 is being filled), so a step
+// needs a single workgroup barrier.
 // -------------------------------------------------------------------------------------------
 constexpr int NT2 = 512;
+constexpr int BQ = 64;   // queries per step of the dk/dv pass
+
+// Experiment-only instrumentation (never defined in the shipped build): thread 0 of each role
+// accumulates shader-clock time per phase into the spare words of the schedule header.
+#ifdef SBA_PHASE_TIMING
+#define SBA_PH_DECL long long ph_t0 = clock64(); long long ph_acc[3] = {0, 0, 0};
+#define SBA_PH(i) { const long long ph_t1 = clock64(); ph_acc[i] += ph_t1 - ph_t0; ph_t0 = ph_t1; }
+#define SBA_PH_FLUSH(sched) if ((threadIdx.x & 255) == 0) { \
+    unsigned long long* d = reinterpret_cast<unsigned long long*>(const_cast<int*>(sched) + 4) + 3 * (threadIdx.x >> 8); \
+    for (int i = 0; i < 3; ++i) atomicAdd(d + i, (unsigned long long)ph_acc[i]); }
+#else
+#define SBA_PH_DECL
+#define SBA_PH(i)
+#define SBA_PH_FLUSH(sched)
+#endif
 
 template <int D, bool AC, bool PROD>
 __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   constexpr int KS = D / 16, DB = D / 32;
-  constexpr int NCHQ = BM * (D / 8) / NT2;
-  constexpr int DBW = DB / 2;   // d-blocks per wave in the dk/dv products
-  // Q and dO tiles: row reads (score operands) and transpose reads (dk/dv operands) -> swizzled.
-  __shared__ __attribute__((aligned(16))) unsigned short Qs[BM * D];
-  __shared__ __attribute__((aligned(16))) unsigned short Gs[BM * D];
-  // p and dz staged [query][key]: 16-byte row writes, transpose reads -> swizzled, 64-key rows.
-  __shared__ __attribute__((aligned(16))) unsigned short Ps[BM * BN];
-  __shared__ __attribute__((aligned(16))) unsigned short Zs[BM * BN];
+  constexpr int NPT = NT2 / 2;                 // threads of one role
+  constexpr int NCHQ = BQ * (D / 8) / NPT;     // 16-byte chunks per product thread per tile
+  constexpr int QTILE = BQ * D;    // elements of one Q or dO tile (swizzled, unpadded)
+  constexpr int PTILE = BQ * BN;   // elements of one staged p or dz block [query][key]
+  // Q and dO tiles: row reads (score operands) and transpose reads (dk/dv operands).
+  __shared__ __attribute__((aligned(16))) unsigned short Qs[4 * QTILE];
+  __shared__ __attribute__((aligned(16))) unsigned short Gs[4 * QTILE];
+  // p and dz staged [query][key]: 16-byte row writes, transpose reads.
+  __shared__ __attribute__((aligned(16))) unsigned short Ps[2 * PTILE];
+  __shared__ __attribute__((aligned(16))) unsigned short Zs[2 * PTILE];
 
   const int* sched = a.sched;
   if (sched[SCHED_STATUS] != 0) return;
@@ -207,8 +251,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63, n = lane & 31, h = lane >> 5;
   const int i16 = lane & 15, blk = (lane >> 4) & 1;
-  const int qg = w >> 1, sb = w & 1;
-  const int k0 = kt * BN + 32 * sb;
+  const bool scorer = w < 4;
 
   const int64_t tok0 = t.tok_start;
   const __bf16* qb = reinterpret_cast<const __bf16*>(a.q.ptr) + t.batch * a.q.sb + head * a.q.sh + tok0 * a.q.st;
@@ -222,111 +265,216 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   const Rows krows = make_rows(kb, a.k.st, t.doc_len);
   const Rows vrows = make_rows(vb, a.v.st, t.doc_len);
 
-  // K and V A-operand fragments of this wave's 32 keys: MFMA row n holds key k0 + kperm(n).
-  bf16x8 kf[KS], vf[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    kf[ks] = load_frag(krows, k0 + kperm(n), 32 * ks + 16 * h);
-    vf[ks] = load_frag(vrows, k0 + kperm(n), 32 * ks + 16 * h);
-  }
+  const int q_first = kt * BN;                                   // first query that can see the tile
+  const int nsteps = (t.doc_len - q_first + BQ - 1) / BQ;        // >= 1
 
-  // Output ownership in the products: matrix (dv / dk), 32-key block, pair of d-blocks.
-  const int mat = w >> 2, kb32 = (w >> 1) & 1, dbp = w & 1;
-  f32x16 acc[DBW];
+  // The two roles run separate copies of the step loop (same barrier count) so that neither
+  // carries the other's registers.
+  // The product waves issue few instructions (16 MFMAs and their operand reads per step) but
+  // each MFMA occupies the matrix core for 8 passes: give them issue priority over the score
+  // waves, whose long VALU streams would otherwise starve them and serialise the two roles.
+  if (scorer) {
+    __builtin_amdgcn_s_setprio(0);
+    const int qg = (w >> 1) & 1, sb = w & 1;
+    const int k0 = kt * BN + 32 * sb;
+    const int qr = 32 * qg + n;                 // this lane's query row inside a tile
+    bf16x8 kf[KS], vf[KS];                      // MFMA row n holds key k0 + kperm(n)
 #pragma unroll
-  for (int j = 0; j < DBW; ++j)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[j][i] = 0.0f;
-  const unsigned short* Xs = mat ? Zs : Ps;   // dz^T or p^T as the A operand
-  const unsigned short* Ys = mat ? Qs : Gs;   // Q or dO as the B operand
-
-  // Transpose-read offsets (elements).  Rows are queries 16*ks + 8*h + 4*u + i/4; the swizzle
-  // depends on the row modulo 16 only, so it is the same for every ks.
-  int xoff[2], yoff[2][DBW];
-#pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    const int r = 8 * h + 4 * u + (i16 >> 2);
-    const int xc = 32 * kb32 + 16 * blk + 4 * (i16 & 3);          // key column (elements)
-    xoff[u] = swz_off<BN>(r, xc >> 3) + (xc & 7);
-#pragma unroll
-    for (int j = 0; j < DBW; ++j) {
-      const int yc = 32 * (DBW * dbp + j) + 16 * blk + 4 * (i16 & 3);   // d column (elements)
-      yoff[u][j] = swz_off<D>(r, yc >> 3) + (yc & 7);
+    for (int ks = 0; ks < KS; ++ks) {
+      kf[ks] = load_frag(krows, k0 + kperm(n), 32 * ks + 16 * h);
+      vf[ks] = load_frag(vrows, k0 + kperm(n), 32 * ks + 16 * h);
     }
-  }
-  // Row-read offsets of this lane's query row for the score operands (chunk 2*ks + h).
-  const int qr = 32 * qg + n;
-  const int64_t tab_head = (int64_t)head * a.n_tt * a.rows_total + (int64_t)t.batch * a.tokens + tok0;
-  const int64_t tix_sb = (int64_t)(2 * kt + sb) * a.rows_total;
-
-  const int qt_first = (kt * BN) / BM;
-  const int qt_last = (t.doc_len - 1) / BM;
-  uint4 qreg[NCHQ], greg[NCHQ];
-  load_tile<D, BM, NT2, false>(qrows, qt_first * BM, qreg);
-  load_tile<D, BM, NT2, false>(grows, qt_first * BM, greg);
-
-  for (int qt = qt_first; qt <= qt_last; ++qt) {
-    const int m0 = qt * BM;
-    __syncthreads();   // previous step's products have consumed Qs, Gs, Ps, Zs
-    store_tile_swizzled<D, BM, NT2>(Qs, qreg);
-    store_tile_swizzled<D, BM, NT2>(Gs, greg);
-    __syncthreads();
-    if (qt < qt_last) {
-      load_tile<D, BM, NT2, false>(qrows, m0 + BM, qreg);
-      load_tile<D, BM, NT2, false>(grows, m0 + BM, greg);
-    }
-
-    const int qw0 = m0 + 32 * qg;
-    const int qrow = qw0 + n;
-    bf16x8 pf[2], zf[2];
-    if (sub_skip<AC>(k0, qw0)) {
-      pf[0] = zero8(); pf[1] = zero8(); zf[0] = zero8(); zf[1] = zero8();
-    } else {
-      f32x16 x, da;
+    const int64_t tab = (int64_t)head * a.n_tt * a.rows_total + (int64_t)t.batch * a.tokens + tok0 +
+                        (int64_t)(2 * kt + sb) * a.rows_total;
+    // per-row carries of a step (neutral past the end of the document)
+    auto carries = [&](int step, float& ce, float& cc, float& d_r) {
+      ce = PROD ? 1.0f : 0.0f; cc = 0.0f; d_r = 0.0f;
+      const int qrow = q_first + step * BQ + qr;
+      if (step < nsteps && qrow < t.doc_len) {
+        ce = a.stick[tab + qrow];
+        cc = a.gtab[tab + qrow];
+        if (grb != nullptr) d_r = (float)grb[(int64_t)qrow * a.grem.st];
+      }
+    };
+    // The row-read offsets of this lane inside a tile (chunk 2*ks + h of row qr).
+    int roff[KS];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) { x[i] = 0.0f; da[i] = 0.0f; }
+    for (int ks = 0; ks < KS; ++ks) roff[ks] = swz_off<D>(qr, 2 * ks + h);
+    auto chains = [&](int slot4, f32x16& x, f32x16& da) {
+      const unsigned short* Qt = Qs + slot4 * QTILE;
+      const unsigned short* Gt = Gs + slot4 * QTILE;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) { x[j] = 0.0f; da[j] = 0.0f; }
+      // all operand reads first, so the chains are not paced by LDS latency
+      bf16x8 qfr[KS], gfr[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) { qfr[ks] = lds_row8(Qt + roff[ks]); gfr[ks] = lds_row8(Gt + roff[ks]); }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        x = mfma32(kf[ks], lds_row8(Qs + swz_off<D>(qr, 2 * ks + h)), x);
-        da = mfma32(vf[ks], lds_row8(Gs + swz_off<D>(qr, 2 * ks + h)), da);
+        x = mfma32(kf[ks], qfr[ks], x);
+        da = mfma32(vf[ks], gfr[ks], da);
       }
-      float carry_e = PROD ? 1.0f : 0.0f, carry_c = 0.0f, dr = 0.0f;
-      if (qrow < t.doc_len) {
-        carry_e = a.stick[tab_head + qrow + tix_sb];
-        carry_c = a.gtab[tab_head + qrow + tix_sb];
-        if (grb != nullptr) dr = (float)grb[(int64_t)qrow * a.grem.st];
+    };
+    auto stage = [&](int step, const bf16x8 (&pf)[2], const bf16x8 (&zf)[2]) {
+      // p and dz as [query][key]: fragment tt is 8 consecutive keys = one 16-byte chunk
+      unsigned short* Pt = Ps + (step & 1) * PTILE;
+      unsigned short* Zt = Zs + (step & 1) * PTILE;
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const int chunk = 4 * sb + 2 * h + tt;
+        *reinterpret_cast<bf16x8*>(Pt + swz_off<BN>(qr, chunk)) = pf[tt];
+        *reinterpret_cast<bf16x8*>(Zt + swz_off<BN>(qr, chunk)) = zf[tt];
       }
-      grad_block<AC, PROD, true>(x, da, a.c, k0, qw0, qrow, h, carry_e, carry_c, dr, pf, zf);
-    }
-    // stage p and dz as [query][key]: fragment tt is 8 consecutive keys = one 16-byte chunk
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-      const int chunk = 4 * sb + 2 * h + tt;
-      *reinterpret_cast<bf16x8*>(Ps + swz_off<BN>(qr, chunk)) = pf[tt];
-      *reinterpret_cast<bf16x8*>(Zs + swz_off<BN>(qr, chunk)) = zf[tt];
-    }
-    __syncthreads();
-    // acc[key, d] += sum over the 128 queries of X[query][key] * Y[query][d]
-#pragma unroll
-    for (int ks = 0; ks < BM / 16; ++ks) {
-      const bf16x8 af = lds_tr8(Xs + xoff[0] + 16 * ks * BN, Xs + xoff[1] + 16 * ks * BN);
-#pragma unroll
-      for (int j = 0; j < DBW; ++j) {
-        const bf16x8 bf = lds_tr8(Ys + yoff[0][j] + 16 * ks * D, Ys + yoff[1][j] + 16 * ks * D);
-        acc[j] = mfma32(af, bf, acc[j]);
-      }
-    }
-  }
+    };
 
-  const View& ov = mat ? a.dk : a.dv;
-  __bf16* outb = reinterpret_cast<__bf16*>(ov.ptr) + t.batch * ov.sb + head * ov.sh + tok0 * ov.st;
-  const float scale = mat ? a.inv_temp : 1.0f;
+    float carry_e, carry_c, dr, ncarry_e, ncarry_c, ndr;
+    carries(0, carry_e, carry_c, dr);
+    carries(1, ncarry_e, ncarry_c, ndr);
+    lds_barrier();                        // tiles 0 and 1 are in slots 0 and 1
+    // One step: (xc, dc) hold the finished chains of block i; the chains of block i+1 go into
+    // (xn, dn).  Called with the two accumulator pairs swapped on alternate steps, so nothing
+    // is copied between steps.
+    auto step = [&](int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn) {
+      // carries of step i+2: requested first, consumed (copied) only after the barrier
+      float e2, c2, r2;
+      carries(i + 2, e2, c2, r2);
+      // MFMA chains of block i+1 (independent of everything below) ...
+#ifndef SBA_X_NO_CHAINS
+      chains((i + 1) & 3, xn, dn);
+#endif
+      // ... while the VALU turns block i into p and dz.
+      bf16x8 pf[2], zf[2];
+      const int qw0 = q_first + i * BQ + 32 * qg;
+      const int qrow = qw0 + n;
+#ifdef SBA_X_NO_VALU
+      if (true) {
+#else
+      if (i == 0 && sub_skip<AC>(k0, qw0)) {
+#endif
+        pf[0] = zero8(); pf[1] = zero8(); zf[0] = zero8(); zf[1] = zero8();
+      } else {
+        float p[16], bt[16];
+        // only the first step can touch the causal diagonal
+        if (i == 0) grad_weights<AC, PROD>(xc, a.c, k0, qw0, qrow, h, carry_e, p, bt);
+        else stick_weights<AC, PROD, false, true>(xc, a.c, k0, qrow, h, carry_e, p, bt);
+        pf[0] = pack8(p);
+        pf[1] = pack8(p + 8);
+        grad_dz(p, bt, dc, h, carry_c, dr, zf);
+      }
+      stage(i, pf, zf);
+      lds_barrier();
+      carry_e = ncarry_e; carry_c = ncarry_c; dr = ndr;
+      ncarry_e = e2; ncarry_c = c2; ndr = r2;
+    };
+    f32x16 xa, da, xb, db;
+    chains(0, xa, da);
+    int i = 0;
+    for (; i + 1 < nsteps; i += 2) {
+      step(i, xa, da, xb, db);
+      step(i + 1, xb, db, xa, da);
+    }
+    if (i < nsteps) step(i, xa, da, xb, db);
+    lds_barrier();                        // the product waves' last step
+  } else {
+    __builtin_amdgcn_s_setprio(3);
+    const int ptid = tid - NPT;
+    const int mat = (w >> 1) & 1, kb32 = w & 1;   // (dv | dk) x 32-key block; all D columns
+    f32x16 acc[DB];
 #pragma unroll
-  for (int j = 0; j < DBW; ++j) {
+    for (int j = 0; j < DB; ++j)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int key = kt * BN + 32 * kb32 + 8 * (i >> 2) + 4 * h + (i & 3);
-      if (key < t.doc_len) outb[(int64_t)key * ov.st + 32 * (DBW * dbp + j) + n] = (__bf16)(acc[j][i] * scale);
+      for (int i = 0; i < 16; ++i) acc[j][i] = 0.0f;
+    // Transpose-read offsets (elements).  Rows are queries 16*ks + 8*h + 4*u + i/4; the swizzle
+    // depends on the row modulo 16 only, so one offset serves every ks.
+    int xoff[2], yoff[2][DB];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int r = 8 * h + 4 * u + (i16 >> 2);
+      const int xc = 32 * kb32 + 16 * blk + 4 * (i16 & 3);          // key column (elements)
+      xoff[u] = swz_off<BN>(r, xc >> 3) + (xc & 7);
+#pragma unroll
+      for (int j = 0; j < DB; ++j) {
+        const int yc = 32 * j + 16 * blk + 4 * (i16 & 3);           // d column (elements)
+        yoff[u][j] = swz_off<D>(r, yc >> 3) + (yc & 7);
+      }
+    }
+    // Tile staging by the 256 product threads: chunk c of a tile -> row c / (D/8).
+    auto fetch = [&](int step, uint4 (&qreg)[NCHQ], uint4 (&greg)[NCHQ]) {
+#pragma unroll
+      for (int j = 0; j < NCHQ; ++j) {
+        const int cidx = ptid + NPT * j;
+        qreg[j] = load16(qrows, q_first + step * BQ + cidx / (D / 8), (cidx % (D / 8)) * 16);
+        greg[j] = load16(grows, q_first + step * BQ + cidx / (D / 8), (cidx % (D / 8)) * 16);
+      }
+    };
+    auto put = [&](int slot4, const uint4 (&qreg)[NCHQ], const uint4 (&greg)[NCHQ]) {
+#pragma unroll
+      for (int j = 0; j < NCHQ; ++j) {
+        const int cidx = ptid + NPT * j;
+        const int off = swz_off<D>(cidx / (D / 8), cidx % (D / 8));
+        *reinterpret_cast<uint4*>(Qs + slot4 * QTILE + off) = qreg[j];
+        *reinterpret_cast<uint4*>(Gs + slot4 * QTILE + off) = greg[j];
+      }
+    };
+    uint4 qa[NCHQ], ga[NCHQ], qb2[NCHQ], gb2[NCHQ];   // two tiles in flight (even / odd steps)
+    fetch(0, qa, ga);
+    fetch(1, qb2, gb2);
+    put(0, qa, ga);
+    put(1, qb2, gb2);
+    fetch(2, qa, ga);
+    fetch(3, qb2, gb2);
+    lds_barrier();
+    SBA_PH_DECL
+    for (int i = 0; i <= nsteps; ++i) {
+      // tile i+2 (requested two steps ago) into its slot, then request tile i+4
+#ifndef SBA_X_NO_STAGE
+      if (i & 1) { put((i + 2) & 3, qb2, gb2); fetch(i + 4, qb2, gb2); }
+      else       { put((i + 2) & 3, qa, ga);   fetch(i + 4, qa, ga); }
+#endif
+      SBA_PH(0)
+#ifdef SBA_X_NO_PRODUCTS
+      if (false) {
+#else
+      if (i >= 1) {
+#endif
+        // acc[key, d] += sum over the 64 queries of step i-1 of X[query][key] * Y[query][d]
+        const unsigned short* Xt = (mat ? Zs : Ps) + ((i - 1) & 1) * PTILE;
+        const unsigned short* Yt = (mat ? Qs : Gs) + ((i - 1) & 3) * QTILE;
+#pragma unroll
+        for (int kh = 0; kh < BQ / 32; ++kh) {
+          // operand reads of two contraction steps first, then their 2*DB products
+          bf16x8 af[2], bf[2][DB];
+#pragma unroll
+          for (int k2 = 0; k2 < 2; ++k2) {
+            const int ks = 2 * kh + k2;
+            af[k2] = lds_tr8(Xt + xoff[0] + 16 * ks * BN, Xt + xoff[1] + 16 * ks * BN);
+#pragma unroll
+            for (int j = 0; j < DB; ++j)
+              bf[k2][j] = lds_tr8(Yt + yoff[0][j] + 16 * ks * D, Yt + yoff[1][j] + 16 * ks * D);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+            for (int j = 0; j < DB; ++j) acc[j] = mfma32(af[k2], bf[k2][j], acc[j]);
+        }
+      }
+      SBA_PH(1)
+      lds_barrier();
+      SBA_PH(2)
+    }
+    SBA_PH_FLUSH(a.sched)
+    const View& ov = mat ? a.dk : a.dv;
+    __bf16* outb = reinterpret_cast<__bf16*>(ov.ptr) + t.batch * ov.sb + head * ov.sh + tok0 * ov.st;
+    const float scale = mat ? a.inv_temp : 1.0f;
+#pragma unroll
+    for (int j = 0; j < DB; ++j) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = kt * BN + 32 * kb32 + 8 * (i >> 2) + 4 * h + (i & 3);
+        if (key < t.doc_len) outb[(int64_t)key * ov.st + 32 * j + n] = (__bf16)(acc[j][i] * scale);
+      }
     }
   }
 }

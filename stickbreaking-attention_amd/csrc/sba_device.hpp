@@ -45,6 +45,14 @@ struct View {
   int64_t sb, sh, st;  // element strides
 };
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every
+// outstanding GLOBAL load (s_waitcnt vmcnt(0)), which would expose the full latency of the
+// tile prefetches and table reads that are deliberately kept in flight across the barrier.
+// The compiler still waits for each load's result before its first use.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
@@ -174,19 +182,24 @@ __device__ __forceinline__ void stick_weights(const f32x16& x, float c, int k0, 
   // visible keys of a band sub-block: key < qrow (<= with attend_current)  <=>  i < lim
   const int lim = qrow - k0 - 16 * h + (AC ? 1 : 0);
   if constexpr (PROD) {
-    float r[16], b[16], ex[16];
+    // r = 1 - beta.  With ex[i] = stick left after the keys newer than key(i), the stick left
+    // after key(i) itself is ex[i] * r[i] = ex[i-1], so the weight is a difference of
+    // consecutive chain values: p[i] = ex[i] - ex[i-1].  A masked key has r = 1, which makes
+    // its p and beta vanish without further masking.
+    float r[16], ex[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
-      const float e = fast_exp2(c * x[i]);   // overflow -> inf -> r = 0, b = 1: still right
-      r[i] = fast_rcp(1.0f + e);             // 1 - beta
-      b[i] = 1.0f - r[i];
-      if (BAND && !(i < lim)) { r[i] = 1.0f; b[i] = 0.0f; }
+      const float e = fast_exp2(c * x[i]);   // overflow -> inf -> r = 0, beta = 1: still right
+      r[i] = fast_rcp(1.0f + e);
+      if (BAND && !(i < lim)) r[i] = 1.0f;
     }
     carry = suffix_prod32_excl(r, ex, h, carry);
+    p[0] = ex[0] - ex[0] * r[0];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      p[i] = b[i] * ex[i];
-      if (NEED_BETA) beta[i] = b[i];
+    for (int i = 1; i < 16; ++i) p[i] = ex[i] - ex[i - 1];
+    if (NEED_BETA) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) beta[i] = 1.0f - r[i];
     }
   } else {
     float xs[16], sp[16];

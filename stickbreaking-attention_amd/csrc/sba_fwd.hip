@@ -69,10 +69,10 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
   load_tile<D, BN, NT, true>(vrows, kt_last * BN, vreg);
 
   for (int kt = kt_last; kt >= 0; --kt) {
-    __syncthreads();
+    lds_barrier();
     store_tile_padded<D, BN, NT, KROW>(Ks, kreg);
     store_tile_padded<D, BN, NT, VROW>(Vs, vreg);
-    __syncthreads();
+    lds_barrier();
     if (kt > 0) {
       load_tile<D, BN, NT, true>(krows, (kt - 1) * BN, kreg);
       load_tile<D, BN, NT, true>(vrows, (kt - 1) * BN, vreg);
@@ -86,9 +86,14 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
       f32x16 x;
 #pragma unroll
       for (int i = 0; i < 16; ++i) x[i] = 0.0f;
+      {
+        // all operand reads first, so the chain is not paced by LDS latency
+        bf16x8 kfr[KS];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        x = mfma32(lds_row8(Ks + (32 * sb + n) * KROW + 16 * ks + 8 * h), qf[ks], x);
+        for (int ks = 0; ks < KS; ++ks) kfr[ks] = lds_row8(Ks + (32 * sb + n) * KROW + 16 * ks + 8 * h);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) x = mfma32(kfr[ks], qf[ks], x);
       }
       float p[16], unused[16];
       if (sub_full<AC>(k0, qw0)) {
@@ -98,15 +103,18 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
       }
       // P as the A operand of O = P.V: slot s of step tt is key 16*h + 8*tt + s, which the
       // permuted tile keeps in LDS row 16*tt + 8*(s/4) + 4*h + s%4.
+      bf16x8 vfr[2][DB];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const unsigned short* vrow = Vs + vtr + (32 * sb + 16 * tt) * VROW;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) vfr[tt][db] = lds_tr8(vrow + 32 * db, vrow + 8 * VROW + 32 * db);
+      }
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt) {
         const bf16x8 pf = pack8(p + 8 * tt);
-        const unsigned short* vrow = Vs + vtr + (32 * sb + 16 * tt) * VROW;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const bf16x8 vf = lds_tr8(vrow + 32 * db, vrow + 8 * VROW + 32 * db);
-          oacc[db] = mfma32(pf, vf, oacc[db]);
-        }
+        for (int db = 0; db < DB; ++db) oacc[db] = mfma32(pf, vfr[tt][db], oacc[db]);
       }
     }
   }
