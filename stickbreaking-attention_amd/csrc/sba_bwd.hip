@@ -19,6 +19,8 @@
 // Per-score math (upstream sb_varlen_bwd.py:439-453):
 //   G = A * (do.v - drem),  C = inclusive running sum of G over keys,  dz = G - beta * C,
 //   dq = s * dz K,  dk = s * dz^T Q,  dv = A^T do.
+#include <type_traits>
+
 #include "sba_kernels.hpp"
 
 namespace sba {
@@ -58,12 +60,11 @@ __device__ __forceinline__ void grad_dz(const float (&p)[16], const float (&bt)[
 template <int D, bool AC, bool PROD>
 __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   constexpr int KS = D / 16, DB = D / 32;
-  constexpr int KROW = D + 8;    // K, V copies for row reads (operands of the score products)
-  constexpr int TROW = D + 32;   // second K copy for transpose reads (operand of dq)
-  constexpr int NCH = BN * (D / 8) / NT;
-  __shared__ __attribute__((aligned(16))) unsigned short Ks[BN * KROW];
-  __shared__ __attribute__((aligned(16))) unsigned short Kt[BN * TROW];
-  __shared__ __attribute__((aligned(16))) unsigned short Vs[BN * KROW];
+  constexpr int TILE = BN * D;   // elements of one K or V tile (unpadded, swizzled)
+  // K (row reads for the scores, transpose reads for dq) and V (row reads) tiles,
+  // double-buffered, filled by asynchronous global -> LDS copies.
+  __shared__ __attribute__((aligned(16))) unsigned short Ks[2 * TILE];
+  __shared__ __attribute__((aligned(16))) unsigned short Vs[2 * TILE];
 
   const int* sched = a.sched;
   if (sched[SCHED_STATUS] != 0) return;
@@ -92,6 +93,9 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   const Rows krows = make_rows(kb, a.k.st, t.doc_len);
   const Rows vrows = make_rows(vb, a.v.st, t.doc_len);
 
+  async_tile<D, BN, NT, true>(krows, 0, Ks, tid);
+  async_tile<D, BN, NT, true>(vrows, 0, Vs, tid);
+
   bf16x8 qf[KS], dof[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
@@ -113,72 +117,93 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
 
   const int last_key = min(m0 + BM - 1, t.doc_len - 1);
   const int kt_last = last_key / BN;
+  // Offsets (elements) inside a tile: row reads of chunk 2*ks + h of LDS row n, and transpose
+  // reads of rows 8*u + 4*h + i/4 (+ 32*sb + 16*tt), columns 32*db + 16*blk + 4*(i%4).
   const int i16 = lane & 15, blk = (lane >> 4) & 1;
-  const int ktr = (4 * h + (i16 >> 2)) * TROW + 16 * blk + 4 * (i16 & 3);
+  int roff[KS], toff[2][DB];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) roff[ks] = swz_off<D>(n, 2 * ks + h);
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int r = 8 * u + 4 * h + (i16 >> 2);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int col = 32 * db + 16 * blk + 4 * (i16 & 3);
+      toff[u][db] = swz_off<D>(r, col >> 3) + (col & 7);
+    }
+  }
   const int64_t tab0 = (int64_t)head * a.n_tt * a.rows_total + grow;
   const float* stick = a.stick + tab0;
   float* gtab = a.gtab + tab0;
 
-  uint4 kreg[NCH], vreg[NCH];
-  load_tile<D, BN, NT, true>(krows, 0, kreg);
-  load_tile<D, BN, NT, true>(vrows, 0, vreg);
-
-  for (int kt = 0; kt <= kt_last; ++kt) {
-    lds_barrier();
-    store_tile_padded<D, BN, NT, KROW>(Ks, kreg);
-    store_tile_padded<D, BN, NT, TROW>(Kt, kreg);
-    store_tile_padded<D, BN, NT, KROW>(Vs, vreg);
-    lds_barrier();
-    // Table reads go out BEFORE the tile prefetch: loads retire in order, so a table value
-    // requested after the prefetch could only be consumed once the whole prefetch had landed.
-    float ce[2];
+  // stick carries of the two sub-blocks of a tile (neutral where the sub-block is skipped)
+  auto carries = [&](int kt, float (&ce)[2]) {
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
       ce[sb] = PROD ? 1.0f : 0.0f;
-      if (qvalid && !sub_skip<AC>(kt * BN + 32 * sb, qw0)) ce[sb] = stick[(int64_t)(2 * kt + sb) * a.rows_total];
+      if (qvalid && kt <= kt_last && !sub_skip<AC>(kt * BN + 32 * sb, qw0)) ce[sb] = stick[(int64_t)(2 * kt + sb) * a.rows_total];
     }
+  };
+  float ce[2], ce_next[2];
+  carries(0, ce);
+
+  int buf = 0;
+  for (int kt = 0; kt <= kt_last; ++kt) {
+    // tile kt has landed and every wave is done with the tile before it
+    wait_loads<0>();
+    lds_barrier();
+    // the next tile's carries go out before its tile copy; neither is waited for in this step
+    carries(kt + 1, ce_next);
     if (kt < kt_last) {
-      load_tile<D, BN, NT, true>(krows, (kt + 1) * BN, kreg);
-      load_tile<D, BN, NT, true>(vrows, (kt + 1) * BN, vreg);
+      async_tile<D, BN, NT, true>(krows, (kt + 1) * BN, Ks + (buf ^ 1) * TILE, tid);
+      async_tile<D, BN, NT, true>(vrows, (kt + 1) * BN, Vs + (buf ^ 1) * TILE, tid);
     }
+    const unsigned short* Kt = Ks + buf * TILE;
+    const unsigned short* Vt = Vs + buf * TILE;
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
       const int k0 = kt * BN + 32 * sb;
       if (sub_skip<AC>(k0, qw0)) continue;
       const int64_t tix = (int64_t)(2 * kt + sb) * a.rows_total;
-      float carry_e = ce[sb];
       if (qvalid && h == 0) gtab[tix] = carry_c;
       float p[16], bt[16];
       {
         f32x16 x;
 #pragma unroll
         for (int i = 0; i < 16; ++i) x[i] = 0.0f;
+        bf16x8 kfr[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-          x = mfma32(lds_row8(Ks + (32 * sb + n) * KROW + 16 * ks + 8 * h), qf[ks], x);
-        grad_weights<AC, PROD>(x, a.c, k0, qw0, qrow, h, carry_e, p, bt);
+        for (int ks = 0; ks < KS; ++ks) kfr[ks] = lds_row8(Kt + 32 * sb * D + roff[ks]);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) x = mfma32(kfr[ks], qf[ks], x);
+        grad_weights<AC, PROD>(x, a.c, k0, qw0, qrow, h, ce[sb], p, bt);
       }
       bf16x8 zf[2];
       {
         f32x16 da;
 #pragma unroll
         for (int i = 0; i < 16; ++i) da[i] = 0.0f;
+        bf16x8 vfr[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-          da = mfma32(lds_row8(Vs + (32 * sb + n) * KROW + 16 * ks + 8 * h), dof[ks], da);
+        for (int ks = 0; ks < KS; ++ks) vfr[ks] = lds_row8(Vt + 32 * sb * D + roff[ks]);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) da = mfma32(vfr[ks], dof[ks], da);
         grad_dz(p, bt, da, h, carry_c, dr, zf);
       }
       // dq += dz . K  (K as the B operand: transpose reads along keys)
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt) {
-        const unsigned short* krow = Kt + ktr + (32 * sb + 16 * tt) * TROW;
+        const unsigned short* krow = Kt + (32 * sb + 16 * tt) * D;
+        bf16x8 kfr[DB];
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const bf16x8 kf = lds_tr8(krow + 32 * db, krow + 8 * TROW + 32 * db);
-          dqacc[db] = mfma32(zf[tt], kf, dqacc[db]);
-        }
+        for (int db = 0; db < DB; ++db) kfr[db] = lds_tr8(krow + toff[0][db], krow + toff[1][db]);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) dqacc[db] = mfma32(zf[tt], kfr[db], dqacc[db]);
       }
     }
+    buf ^= 1;
+    ce[0] = ce_next[0];
+    ce[1] = ce_next[1];
   }
 
 #pragma unroll
@@ -229,7 +254,6 @@ template <int D, bool AC, bool PROD>
 __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   constexpr int KS = D / 16, DB = D / 32;
   constexpr int NPT = NT2 / 2;                 // threads of one role
-  constexpr int NCHQ = BQ * (D / 8) / NPT;     // 16-byte chunks per product thread per tile
   constexpr int QTILE = BQ * D;    // elements of one Q or dO tile (swizzled, unpadded)
   constexpr int PTILE = BQ * BN;   // elements of one staged p or dz block [query][key]
   // Q and dO tiles: row reads (score operands) and transpose reads (dk/dv operands).
@@ -286,15 +310,20 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     }
     const int64_t tab = (int64_t)head * a.n_tt * a.rows_total + (int64_t)t.batch * a.tokens + tok0 +
                         (int64_t)(2 * kt + sb) * a.rows_total;
-    // per-row carries of a step (neutral past the end of the document)
+    // per-row carries of a step, branch-free: the address is clamped into the document and the
+    // value replaced by the neutral element past its end (those rows have zero Q and dO)
+    const int64_t grem_st = grb != nullptr ? a.grem.st : 0;
+    const __bf16* grb_safe = grb != nullptr ? grb : reinterpret_cast<const __bf16*>(a.stick);
     auto carries = [&](int step, float& ce, float& cc, float& d_r) {
-      ce = PROD ? 1.0f : 0.0f; cc = 0.0f; d_r = 0.0f;
       const int qrow = q_first + step * BQ + qr;
-      if (step < nsteps && qrow < t.doc_len) {
-        ce = a.stick[tab + qrow];
-        cc = a.gtab[tab + qrow];
-        if (grb != nullptr) d_r = (float)grb[(int64_t)qrow * a.grem.st];
-      }
+      const bool ok = qrow < t.doc_len;
+      const int qc = ok ? qrow : t.doc_len - 1;
+      const float e = a.stick[tab + qc];
+      const float g = a.gtab[tab + qc];
+      const float d = (float)grb_safe[(int64_t)qc * grem_st];
+      ce = ok ? e : (PROD ? 1.0f : 0.0f);
+      cc = ok ? g : 0.0f;
+      d_r = (ok && grb != nullptr) ? d : 0.0f;
     };
     // The row-read offsets of this lane inside a tile (chunk 2*ks + h of row qr).
     int roff[KS];
@@ -309,7 +338,6 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       bf16x8 qfr[KS], gfr[KS];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) { qfr[ks] = lds_row8(Qt + roff[ks]); gfr[ks] = lds_row8(Gt + roff[ks]); }
-      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         x = mfma32(kf[ks], qfr[ks], x);
@@ -334,47 +362,50 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     lds_barrier();                        // tiles 0 and 1 are in slots 0 and 1
     // One step: (xc, dc) hold the finished chains of block i; the chains of block i+1 go into
     // (xn, dn).  Called with the two accumulator pairs swapped on alternate steps, so nothing
-    // is copied between steps.
-    auto step = [&](int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn) {
+    // is copied between steps.  FIRST = the step on the causal diagonal (masks, possible skip);
+    // every later step is one straight-line block in which the MFMA chains of block i+1 are
+    // interleaved with the VALU work on block i.
+    auto step = [&](auto first_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn) {
+      constexpr bool FIRST = decltype(first_tag)::value;
       // carries of step i+2: requested first, consumed (copied) only after the barrier
       float e2, c2, r2;
       carries(i + 2, e2, c2, r2);
-      // MFMA chains of block i+1 (independent of everything below) ...
-#ifndef SBA_X_NO_CHAINS
       chains((i + 1) & 3, xn, dn);
-#endif
-      // ... while the VALU turns block i into p and dz.
       bf16x8 pf[2], zf[2];
       const int qw0 = q_first + i * BQ + 32 * qg;
       const int qrow = qw0 + n;
-#ifdef SBA_X_NO_VALU
-      if (true) {
-#else
-      if (i == 0 && sub_skip<AC>(k0, qw0)) {
-#endif
+      if (FIRST && sub_skip<AC>(k0, qw0)) {
         pf[0] = zero8(); pf[1] = zero8(); zf[0] = zero8(); zf[1] = zero8();
       } else {
         float p[16], bt[16];
-        // only the first step can touch the causal diagonal
-        if (i == 0) grad_weights<AC, PROD>(xc, a.c, k0, qw0, qrow, h, carry_e, p, bt);
+        if (FIRST) grad_weights<AC, PROD>(xc, a.c, k0, qw0, qrow, h, carry_e, p, bt);
         else stick_weights<AC, PROD, false, true>(xc, a.c, k0, qrow, h, carry_e, p, bt);
         pf[0] = pack8(p);
         pf[1] = pack8(p + 8);
         grad_dz(p, bt, dc, h, carry_c, dr, zf);
       }
       stage(i, pf, zf);
+      if (!FIRST) {
+        // operand reads first, then one MFMA per group of VALU instructions
+#pragma unroll
+        for (int g = 0; g < 2 * KS; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x006, 96 / KS, 0);
+        }
+      }
       lds_barrier();
       carry_e = ncarry_e; carry_c = ncarry_c; dr = ndr;
       ncarry_e = e2; ncarry_c = c2; ndr = r2;
     };
     f32x16 xa, da, xb, db;
     chains(0, xa, da);
-    int i = 0;
+    step(std::true_type{}, 0, xa, da, xb, db);
+    int i = 1;
     for (; i + 1 < nsteps; i += 2) {
-      step(i, xa, da, xb, db);
-      step(i + 1, xb, db, xa, da);
+      step(std::false_type{}, i, xb, db, xa, da);
+      step(std::false_type{}, i + 1, xa, da, xb, db);
     }
-    if (i < nsteps) step(i, xa, da, xb, db);
+    if (i < nsteps) step(std::false_type{}, i, xb, db, xa, da);
     lds_barrier();                        // the product waves' last step
   } else {
     __builtin_amdgcn_s_setprio(3);
@@ -399,38 +430,20 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
         yoff[u][j] = swz_off<D>(r, yc >> 3) + (yc & 7);
       }
     }
-    // Tile staging by the 256 product threads: chunk c of a tile -> row c / (D/8).
-    auto fetch = [&](int step, uint4 (&qreg)[NCHQ], uint4 (&greg)[NCHQ]) {
-#pragma unroll
-      for (int j = 0; j < NCHQ; ++j) {
-        const int cidx = ptid + NPT * j;
-        qreg[j] = load16(qrows, q_first + step * BQ + cidx / (D / 8), (cidx % (D / 8)) * 16);
-        greg[j] = load16(grows, q_first + step * BQ + cidx / (D / 8), (cidx % (D / 8)) * 16);
-      }
+    // Tile staging by the 256 product threads: asynchronous global -> LDS copies straight into
+    // the ring slot, one step ahead of the score waves that will read it.
+    auto fetch = [&](int step) {
+      async_tile<D, BQ, NPT, false>(qrows, q_first + step * BQ, Qs + (step & 3) * QTILE, ptid);
+      async_tile<D, BQ, NPT, false>(grows, q_first + step * BQ, Gs + (step & 3) * QTILE, ptid);
     };
-    auto put = [&](int slot4, const uint4 (&qreg)[NCHQ], const uint4 (&greg)[NCHQ]) {
-#pragma unroll
-      for (int j = 0; j < NCHQ; ++j) {
-        const int cidx = ptid + NPT * j;
-        const int off = swz_off<D>(cidx / (D / 8), cidx % (D / 8));
-        *reinterpret_cast<uint4*>(Qs + slot4 * QTILE + off) = qreg[j];
-        *reinterpret_cast<uint4*>(Gs + slot4 * QTILE + off) = greg[j];
-      }
-    };
-    uint4 qa[NCHQ], ga[NCHQ], qb2[NCHQ], gb2[NCHQ];   // two tiles in flight (even / odd steps)
-    fetch(0, qa, ga);
-    fetch(1, qb2, gb2);
-    put(0, qa, ga);
-    put(1, qb2, gb2);
-    fetch(2, qa, ga);
-    fetch(3, qb2, gb2);
+    fetch(0);
+    fetch(1);
+    wait_loads<0>();
     lds_barrier();
     SBA_PH_DECL
     for (int i = 0; i <= nsteps; ++i) {
-      // tile i+2 (requested two steps ago) into its slot, then request tile i+4
 #ifndef SBA_X_NO_STAGE
-      if (i & 1) { put((i + 2) & 3, qb2, gb2); fetch(i + 4, qb2, gb2); }
-      else       { put((i + 2) & 3, qa, ga);   fetch(i + 4, qa, ga); }
+      if (i + 2 < nsteps) fetch(i + 2);
 #endif
       SBA_PH(0)
 #ifdef SBA_X_NO_PRODUCTS
@@ -461,6 +474,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
         }
       }
       SBA_PH(1)
+      wait_loads<0>();   // tile i+2 has landed before anyone passes the barrier
       lds_barrier();
       SBA_PH(2)
     }

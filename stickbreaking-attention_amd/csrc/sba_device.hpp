@@ -303,6 +303,39 @@ __device__ __forceinline__ int swz_off(int row, int chunk) {   // element offset
   return row * D + ((chunk ^ swz<D>(row)) << 3);
 }
 
+// Asynchronous global -> LDS copy of ROWS x D bf16 of a (document, head) slice into an unpadded,
+// swizzled tile, issued by the THREADS threads whose index inside their group is `gtid`
+// (buffer_load_dwordx4 ... lds).  One wave instruction moves 1 KiB: lane l fills the 16-byte
+// LDS chunk number (first chunk of the instruction + l), so the swizzle (and the key
+// permutation of key tiles) is applied on the GLOBAL side by choosing which chunk a lane
+// fetches; rows past the end of the document arrive as zeros.  Completion is tracked by vmcnt:
+// wait for it, then barrier, before any wave reads the tile.
+template <int D, int ROWS, int THREADS, bool KEYS>
+__device__ __forceinline__ void async_tile(const Rows& r, int row0, unsigned short* lds_tile, int gtid) {
+  constexpr int C8 = D / 8;
+  constexpr int NCH = ROWS * C8 / THREADS;
+  static_assert(ROWS * C8 % THREADS == 0, "tile must split evenly over the loading threads");
+  const int wave = __builtin_amdgcn_readfirstlane(gtid >> 6), lane = gtid & 63;
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    const int chunk0 = (wave * NCH + j) * 64;       // wave-uniform
+    const int cidx = chunk0 + lane;
+    const int m = cidx / C8, phys = cidx % C8;
+    const int logical = phys ^ swz<D>(m);
+    const int src = KEYS ? ((m & ~31) | kperm(m & 31)) : m;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(
+        r.rsrc, (__attribute__((address_space(3))) void*)(lds_tile + chunk0 * 8), 16,
+        (row0 + src) * (int)r.row_bytes + logical * 16, 0, 0, 0);
+  }
+}
+
+// Wait until at most N of this wave's global loads (including asynchronous tile copies) are
+// still in flight.
+template <int N>
+__device__ __forceinline__ void wait_loads() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
 template <int D, int ROWS, int THREADS>
 __device__ __forceinline__ void store_tile_swizzled(unsigned short* lds, const uint4 (&reg)[ROWS * (D / 8) / THREADS]) {
   constexpr int C8 = D / 8;

@@ -12,11 +12,10 @@ template <int D, bool AC, bool PROD>
 __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
   constexpr int KS = D / 16;     // contraction steps of K.Q^T
   constexpr int DB = D / 32;     // 32-wide output column blocks of P.V
-  constexpr int KROW = D + 8;    // K tile: row (b128) reads, stride = 4 banks mod 64
-  constexpr int VROW = D + 32;   // V tile: transpose reads, stride = 16 banks mod 64
-  constexpr int NCH = BN * (D / 8) / NT;
-  __shared__ __attribute__((aligned(16))) unsigned short Ks[BN * KROW];
-  __shared__ __attribute__((aligned(16))) unsigned short Vs[BN * VROW];
+  constexpr int TILE = BN * D;   // elements of one K or V tile (unpadded, swizzled)
+  // K and V tiles, double-buffered, filled by asynchronous global -> LDS copies.
+  __shared__ __attribute__((aligned(16))) unsigned short Ks[2 * TILE];
+  __shared__ __attribute__((aligned(16))) unsigned short Vs[2 * TILE];
 
   const int* sched = a.sched;
   if (sched[SCHED_STATUS] != 0) return;
@@ -44,6 +43,11 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
   const Rows krows = make_rows(kb, a.k.st, t.doc_len);
   const Rows vrows = make_rows(vb, a.v.st, t.doc_len);
 
+  const int last_key = min(m0 + BM - 1, t.doc_len - 1);
+  const int kt_last = last_key / BN;
+  async_tile<D, BN, NT, true>(krows, kt_last * BN, Ks, tid);
+  async_tile<D, BN, NT, true>(vrows, kt_last * BN, Vs, tid);
+
   // Q^T operand fragments: lane (n, h) holds Q[qrow][16*ks + 8*h .. +7] (zeros past the document).
   bf16x8 qf[KS];
 #pragma unroll
@@ -56,27 +60,34 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
     for (int i = 0; i < 16; ++i) oacc[db][i] = 0.0f;
   float carry = PROD ? 1.0f : 0.0f;
 
-  const int last_key = min(m0 + BM - 1, t.doc_len - 1);
-  const int kt_last = last_key / BN;
-
-  // per-lane offset for the transpose reads of V: row 4*h + i/4, column 16*blk + 4*(i%4)
+  // Offsets (elements) inside a tile.  K: row read of chunk 2*ks + h of LDS row n (= MFMA row n).
+  // V: transpose reads of rows 8*u + 4*h + i/4 (+ 32*sb + 16*tt), columns 32*db + 16*blk + 4*(i%4).
   const int i16 = lane & 15, blk = (lane >> 4) & 1;
-  const int vtr = (4 * h + (i16 >> 2)) * VROW + 16 * blk + 4 * (i16 & 3);
+  int koff[KS], voff[2][DB];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) koff[ks] = swz_off<D>(n, 2 * ks + h);
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int r = 8 * u + 4 * h + (i16 >> 2);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int col = 32 * db + 16 * blk + 4 * (i16 & 3);
+      voff[u][db] = swz_off<D>(r, col >> 3) + (col & 7);
+    }
+  }
   float* stick = a.stick == nullptr ? nullptr : a.stick + (int64_t)head * a.n_tt * a.rows_total + grow;
 
-  uint4 kreg[NCH], vreg[NCH];
-  load_tile<D, BN, NT, true>(krows, kt_last * BN, kreg);
-  load_tile<D, BN, NT, true>(vrows, kt_last * BN, vreg);
-
+  int buf = 0;
   for (int kt = kt_last; kt >= 0; --kt) {
-    lds_barrier();
-    store_tile_padded<D, BN, NT, KROW>(Ks, kreg);
-    store_tile_padded<D, BN, NT, VROW>(Vs, vreg);
+    // tile kt has landed and every wave is done with the tile before it
+    wait_loads<0>();
     lds_barrier();
     if (kt > 0) {
-      load_tile<D, BN, NT, true>(krows, (kt - 1) * BN, kreg);
-      load_tile<D, BN, NT, true>(vrows, (kt - 1) * BN, vreg);
+      async_tile<D, BN, NT, true>(krows, (kt - 1) * BN, Ks + (buf ^ 1) * TILE, tid);
+      async_tile<D, BN, NT, true>(vrows, (kt - 1) * BN, Vs + (buf ^ 1) * TILE, tid);
     }
+    const unsigned short* Kt = Ks + buf * TILE;
+    const unsigned short* Vt = Vs + buf * TILE;
 #pragma unroll
     for (int sb = 1; sb >= 0; --sb) {
       const int k0 = kt * BN + 32 * sb;
@@ -87,11 +98,9 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) x[i] = 0.0f;
       {
-        // all operand reads first, so the chain is not paced by LDS latency
         bf16x8 kfr[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) kfr[ks] = lds_row8(Ks + (32 * sb + n) * KROW + 16 * ks + 8 * h);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int ks = 0; ks < KS; ++ks) kfr[ks] = lds_row8(Kt + 32 * sb * D + koff[ks]);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) x = mfma32(kfr[ks], qf[ks], x);
       }
@@ -106,9 +115,9 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
       bf16x8 vfr[2][DB];
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt) {
-        const unsigned short* vrow = Vs + vtr + (32 * sb + 16 * tt) * VROW;
+        const unsigned short* vrow = Vt + (32 * sb + 16 * tt) * D;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) vfr[tt][db] = lds_tr8(vrow + 32 * db, vrow + 8 * VROW + 32 * db);
+        for (int db = 0; db < DB; ++db) vfr[tt][db] = lds_tr8(vrow + voff[0][db], vrow + voff[1][db]);
       }
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt) {
@@ -117,6 +126,7 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
         for (int db = 0; db < DB; ++db) oacc[db] = mfma32(pf, vfr[tt][db], oacc[db]);
       }
     }
+    buf ^= 1;
   }
 
   // epilogue: rem = what is left of the stick; o rows in the accumulator layout
