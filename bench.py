@@ -62,6 +62,8 @@ def main():
     ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--log-space", action="store_true", help="log2-sum carry instead of product carry")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device copy (reference dispatch for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus must be 1", file=sys.stderr)
@@ -98,6 +100,12 @@ def main():
         with torch.no_grad():
             return sb_attn_varlen(q, k, v, cu, max_len, zero_start=cfg["zero_start"])
 
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

@@ -27,8 +27,8 @@ namespace sba {
 
 // One 32-key sub-block for the 32 queries of a wave, in two phases so that the do.v^T
 // accumulators need not be live while the weights are formed:
-//   grad_weights  p, beta from the raw scores and the stick carry at the sub-block's newer edge
-//   grad_dz       G = p (do.v - drem), dz = G - beta C with the running prefix C of G
+//   grad_weights  p and r = 1 - beta from the raw scores and the stick carry at the sub-block's newer edge
+//   grad_dz       dz = G - beta C with G = p (do.v - drem) and the running prefix C of G
 //                 (carry_c: in = prefix before the sub-block, out = after it)
 // p and dz leave as bf16 A-operand fragments: slot s of fragment [tt] is key 16*h + 8*tt + s.
 template <bool AC, bool PROD>
@@ -41,15 +41,30 @@ __device__ __forceinline__ void grad_weights(const f32x16& x, float c, int k0, i
   }
 }
 
-__device__ __forceinline__ void grad_dz(const float (&p)[16], const float (&bt)[16], const f32x16& da, int h,
+// With G = p (do.v - drem), C the inclusive running sum of G along the keys and r = 1 - beta:
+//   dz = G - beta C = r C - (C - G) = r * C[i] - C[i-1],
+// so neither G nor beta is formed: the running sum is an fma chain and dz one more fma.  A
+// masked key has p = 0 and r = 1, which gives dz = 0 exactly.
+__device__ __forceinline__ void grad_dz(const float (&p)[16], const float (&r)[16], const f32x16& da, int h,
                                         float& carry_c, float dr, bf16x8 (&zf)[2]) {
-  float g[16], cs[16];
+  float dA[16];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) { g[i] = p[i] * (da[i] - dr); cs[i] = g[i]; }
-  carry_c += prefix_sum32(cs, h, carry_c);
+  for (int i = 0; i < 16; ++i) dA[i] = da[i] - dr;
+  // this lane's total of G (two partial chains), then both half-waves' totals
+  float t0 = 0.0f, t1 = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 16; i += 2) { t0 = fmaf(p[i], dA[i], t0); t1 = fmaf(p[i + 1], dA[i + 1], t1); }
+  float lo, hi;
+  both_halves(t0 + t1, lo, hi);
+  float cprev = h == 1 ? carry_c + lo : carry_c;   // keys of the h=0 lane come first
   float dz[16];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) dz[i] = g[i] - bt[i] * cs[i];
+  for (int i = 0; i < 16; ++i) {
+    const float c = fmaf(p[i], dA[i], cprev);
+    dz[i] = fmaf(r[i], c, -cprev);
+    cprev = c;
+  }
+  carry_c += lo + hi;
   zf[0] = pack8(dz);
   zf[1] = pack8(dz + 8);
 }
@@ -93,8 +108,11 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   const Rows krows = make_rows(kb, a.k.st, t.doc_len);
   const Rows vrows = make_rows(vb, a.v.st, t.doc_len);
 
-  async_tile<D, BN, NT, true>(krows, 0, Ks, tid);
-  async_tile<D, BN, NT, true>(vrows, 0, Vs, tid);
+  TileCopy<D, BN, NT, true> kcopy, vcopy;
+  kcopy.init(tid, krows.row_bytes);
+  vcopy.init(tid, vrows.row_bytes);
+  kcopy.issue(krows, 0, Ks);
+  vcopy.issue(vrows, 0, Vs);
 
   bf16x8 qf[KS], dof[KS];
 #pragma unroll
@@ -155,8 +173,8 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
     // the next tile's carries go out before its tile copy; neither is waited for in this step
     carries(kt + 1, ce_next);
     if (kt < kt_last) {
-      async_tile<D, BN, NT, true>(krows, (kt + 1) * BN, Ks + (buf ^ 1) * TILE, tid);
-      async_tile<D, BN, NT, true>(vrows, (kt + 1) * BN, Vs + (buf ^ 1) * TILE, tid);
+      kcopy.issue(krows, (kt + 1) * BN, Ks + (buf ^ 1) * TILE);
+      vcopy.issue(vrows, (kt + 1) * BN, Vs + (buf ^ 1) * TILE);
     }
     const unsigned short* Kt = Ks + buf * TILE;
     const unsigned short* Vt = Vs + buf * TILE;
@@ -263,6 +281,9 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   __shared__ __attribute__((aligned(16))) unsigned short Ps[2 * PTILE];
   __shared__ __attribute__((aligned(16))) unsigned short Zs[2 * PTILE];
 
+#ifdef SBA_PHASE_TIMING
+  const long long wg_t0 = clock64();
+#endif
   const int* sched = a.sched;
   if (sched[SCHED_STATUS] != 0) return;
   const int slot = blockIdx.x / a.heads;
@@ -310,20 +331,26 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     }
     const int64_t tab = (int64_t)head * a.n_tt * a.rows_total + (int64_t)t.batch * a.tokens + tok0 +
                         (int64_t)(2 * kt + sb) * a.rows_total;
-    // per-row carries of a step, branch-free: the address is clamped into the document and the
-    // value replaced by the neutral element past its end (those rows have zero Q and dO)
+    // Per-row carries of a step, branch-free: the address is clamped into the document and the
+    // value replaced by the neutral element past its end (those rows have zero Q and dO).
     const int64_t grem_st = grb != nullptr ? a.grem.st : 0;
     const __bf16* grb_safe = grb != nullptr ? grb : reinterpret_cast<const __bf16*>(a.stick);
-    auto carries = [&](int step, float& ce, float& cc, float& d_r) {
+    // `request` only issues the loads; `settle` applies the end-of-document selection.  They are
+    // kept apart so that nothing consumes (and therefore waits for) a loaded value until a
+    // whole step after the request.
+    struct Raw { float e, g; unsigned short d; };   // d: grad_rem still as bf16 bits
+    auto request = [&](int step, Raw& r) {
       const int qrow = q_first + step * BQ + qr;
-      const bool ok = qrow < t.doc_len;
-      const int qc = ok ? qrow : t.doc_len - 1;
-      const float e = a.stick[tab + qc];
-      const float g = a.gtab[tab + qc];
-      const float d = (float)grb_safe[(int64_t)qc * grem_st];
-      ce = ok ? e : (PROD ? 1.0f : 0.0f);
-      cc = ok ? g : 0.0f;
-      d_r = (ok && grb != nullptr) ? d : 0.0f;
+      const int qc = qrow < t.doc_len ? qrow : t.doc_len - 1;
+      r.e = a.stick[tab + qc];
+      r.g = a.gtab[tab + qc];
+      r.d = reinterpret_cast<const unsigned short*>(grb_safe)[(int64_t)qc * grem_st];
+    };
+    auto settle = [&](int step, const Raw& r, float& ce, float& cc, float& d_r) {
+      const bool ok = q_first + step * BQ + qr < t.doc_len;
+      ce = ok ? r.e : (PROD ? 1.0f : 0.0f);
+      cc = ok ? r.g : 0.0f;
+      d_r = (ok && grb != nullptr) ? __builtin_bit_cast(float, (unsigned)r.d << 16) : 0.0f;
     };
     // The row-read offsets of this lane inside a tile (chunk 2*ks + h of row qr).
     int roff[KS];
@@ -356,20 +383,31 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       }
     };
 
+    // Carries are requested three steps ahead and settled two steps ahead, alternating between
+    // two register sets, so a request has two full steps to complete.
     float carry_e, carry_c, dr, ncarry_e, ncarry_c, ndr;
-    carries(0, carry_e, carry_c, dr);
-    carries(1, ncarry_e, ncarry_c, ndr);
+    Raw ra, rb;
+    {
+      Raw r0, r1;
+      request(0, r0);
+      request(1, r1);
+      request(2, rb);
+      settle(0, r0, carry_e, carry_c, dr);
+      settle(1, r1, ncarry_e, ncarry_c, ndr);
+    }
     lds_barrier();                        // tiles 0 and 1 are in slots 0 and 1
+#ifdef SBA_PHASE_TIMING
+    const long long wg_t1 = clock64();
+#endif
     // One step: (xc, dc) hold the finished chains of block i; the chains of block i+1 go into
     // (xn, dn).  Called with the two accumulator pairs swapped on alternate steps, so nothing
     // is copied between steps.  FIRST = the step on the causal diagonal (masks, possible skip);
     // every later step is one straight-line block in which the MFMA chains of block i+1 are
     // interleaved with the VALU work on block i.
-    auto step = [&](auto first_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn) {
+    auto step = [&](auto first_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& req,
+                    const Raw& due) {
       constexpr bool FIRST = decltype(first_tag)::value;
-      // carries of step i+2: requested first, consumed (copied) only after the barrier
-      float e2, c2, r2;
-      carries(i + 2, e2, c2, r2);
+      request(i + 3, req);
       chains((i + 1) & 3, xn, dn);
       bf16x8 pf[2], zf[2];
       const int qw0 = q_first + i * BQ + 32 * qg;
@@ -385,28 +423,117 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
         grad_dz(p, bt, dc, h, carry_c, dr, zf);
       }
       stage(i, pf, zf);
-      if (!FIRST) {
-        // operand reads first, then one MFMA per group of VALU instructions
-#pragma unroll
-        for (int g = 0; g < 2 * KS; ++g) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x006, 96 / KS, 0);
-        }
-      }
       lds_barrier();
+      __builtin_amdgcn_sched_barrier(0);   // keep the consumers of the requested values down here
       carry_e = ncarry_e; carry_c = ncarry_c; dr = ndr;
-      ncarry_e = e2; ncarry_c = c2; ndr = r2;
+      settle(i + 2, due, ncarry_e, ncarry_c, ndr);   // requested one step ago
+    };
+    // The same step for the product-space carry away from the diagonal, hand-pipelined: the
+    // VALU work on block i is cut into 8 chunks and the 2*KS chain MFMAs of block i+1 are
+    // issued between them (operand reads one chunk ahead), each position pinned with a
+    // scheduling barrier so that the matrix core runs underneath the VALU stream.
+    auto bulk = [&](int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& req, const Raw& due) {
+      constexpr int NCHUNK = 8, PER = 2 * KS / NCHUNK;
+      request(i + 3, req);
+      const unsigned short* Qt = Qs + ((i + 1) & 3) * QTILE;
+      const unsigned short* Gt = Gs + ((i + 1) & 3) * QTILE;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) { xn[j] = 0.0f; dn[j] = 0.0f; }
+      bf16x8 fr[PER];
+      auto pre = [&](int c) {
+#pragma unroll
+        for (int m = 0; m < PER; ++m) {
+          const int k = c * PER + m;   // even: q.k chain step k/2, odd: do.v chain step k/2
+          fr[m] = lds_row8(((k & 1) ? Gt : Qt) + roff[k >> 1]);
+        }
+      };
+      auto post = [&](int c) {
+#pragma unroll
+        for (int m = 0; m < PER; ++m) {
+          const int k = c * PER + m;
+          if (k & 1) dn = mfma32(vf[k >> 1], fr[m], dn);
+          else xn = mfma32(kf[k >> 1], fr[m], xn);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      float r[16], ex[16], p[16];
+      // chunks 0, 1: r = 1 - beta of the 16 keys
+      pre(0);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) r[j] = fast_rcp(1.0f + fast_exp2(a.c * xc[j]));
+      post(0);
+      pre(1);
+#pragma unroll
+      for (int j = 8; j < 16; ++j) r[j] = fast_rcp(1.0f + fast_exp2(a.c * xc[j]));
+      post(1);
+      // chunk 2: stick left after the newer keys
+      pre(2);
+      carry_e = suffix_prod32_excl(r, ex, h, carry_e);
+      post(2);
+      // chunk 3: weights and their bf16 fragments
+      pre(3);
+      p[0] = ex[0] - ex[0] * r[0];
+#pragma unroll
+      for (int j = 1; j < 16; ++j) p[j] = ex[j] - ex[j - 1];
+      bf16x8 pf[2], zf[2];
+      pf[0] = pack8(p);
+      pf[1] = pack8(p + 8);
+      post(3);
+      // chunk 4: do.v - drem and this lane's total of G
+      pre(4);
+      float dA[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) dA[j] = dc[j] - dr;
+      float t0 = 0.0f, t1 = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 16; j += 2) { t0 = fmaf(p[j], dA[j], t0); t1 = fmaf(p[j + 1], dA[j + 1], t1); }
+      float lo, hi;
+      both_halves(t0 + t1, lo, hi);
+      float cprev = h == 1 ? carry_c + lo : carry_c;
+      post(4);
+      // chunks 5, 6: running sum of G and dz = r C[i] - C[i-1]
+      float dz[16];
+      pre(5);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) { const float cj = fmaf(p[j], dA[j], cprev); dz[j] = fmaf(r[j], cj, -cprev); cprev = cj; }
+      post(5);
+      pre(6);
+#pragma unroll
+      for (int j = 8; j < 16; ++j) { const float cj = fmaf(p[j], dA[j], cprev); dz[j] = fmaf(r[j], cj, -cprev); cprev = cj; }
+      post(6);
+      // chunk 7: dz fragments and staging
+      pre(7);
+      zf[0] = pack8(dz);
+      zf[1] = pack8(dz + 8);
+      stage(i, pf, zf);
+      post(7);
+      lds_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      carry_c = ncarry_c;   // (the running sum of this step ended in registers only)
+      carry_e = ncarry_e; dr = ndr;
+      settle(i + 2, due, ncarry_e, ncarry_c, ndr);
+    };
+    auto later = [&](int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& req, const Raw& due) {
+      if constexpr (PROD) bulk(i, xc, dc, xn, dn, req, due);
+      else step(std::false_type{}, i, xc, dc, xn, dn, req, due);
     };
     f32x16 xa, da, xb, db;
     chains(0, xa, da);
-    step(std::true_type{}, 0, xa, da, xb, db);
+    step(std::true_type{}, 0, xa, da, xb, db, ra, rb);
     int i = 1;
     for (; i + 1 < nsteps; i += 2) {
-      step(std::false_type{}, i, xb, db, xa, da);
-      step(std::false_type{}, i + 1, xa, da, xb, db);
+      later(i, xb, db, xa, da, rb, ra);
+      later(i + 1, xa, da, xb, db, ra, rb);
     }
-    if (i < nsteps) step(std::false_type{}, i, xb, db, xa, da);
+    if (i < nsteps) later(i, xb, db, xa, da, rb, ra);
     lds_barrier();                        // the product waves' last step
+#ifdef SBA_PHASE_TIMING
+    if (threadIdx.x == 0) {
+      unsigned long long* d = reinterpret_cast<unsigned long long*>(const_cast<int*>(a.sched) + 4);
+      atomicAdd(d + 4, (unsigned long long)(wg_t1 - wg_t0));
+      atomicAdd(d + 5, (unsigned long long)(clock64() - wg_t0));
+    }
+#endif
   } else {
     __builtin_amdgcn_s_setprio(3);
     const int ptid = tid - NPT;
@@ -432,9 +559,12 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     }
     // Tile staging by the 256 product threads: asynchronous global -> LDS copies straight into
     // the ring slot, one step ahead of the score waves that will read it.
+    TileCopy<D, BQ, NPT, false> qcopy, gcopy;
+    qcopy.init(ptid, qrows.row_bytes);
+    gcopy.init(ptid, grows.row_bytes);
     auto fetch = [&](int step) {
-      async_tile<D, BQ, NPT, false>(qrows, q_first + step * BQ, Qs + (step & 3) * QTILE, ptid);
-      async_tile<D, BQ, NPT, false>(grows, q_first + step * BQ, Gs + (step & 3) * QTILE, ptid);
+      qcopy.issue(qrows, q_first + step * BQ, Qs + (step & 3) * QTILE);
+      gcopy.issue(grows, q_first + step * BQ, Gs + (step & 3) * QTILE);
     };
     fetch(0);
     fetch(1);
@@ -492,6 +622,25 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     }
   }
 }
+
+
+// Explicit instantiations: every (head_dim, attend_current, carry space) variant the launchers use.
+template __global__ void bwd_dq_kernel<64, false, false>(const KArgs);
+template __global__ void bwd_dq_kernel<64, false, true>(const KArgs);
+template __global__ void bwd_dq_kernel<64, true, false>(const KArgs);
+template __global__ void bwd_dq_kernel<64, true, true>(const KArgs);
+template __global__ void bwd_dq_kernel<128, false, false>(const KArgs);
+template __global__ void bwd_dq_kernel<128, false, true>(const KArgs);
+template __global__ void bwd_dq_kernel<128, true, false>(const KArgs);
+template __global__ void bwd_dq_kernel<128, true, true>(const KArgs);
+template __global__ void bwd_dkdv_kernel<64, false, false>(const KArgs);
+template __global__ void bwd_dkdv_kernel<64, false, true>(const KArgs);
+template __global__ void bwd_dkdv_kernel<64, true, false>(const KArgs);
+template __global__ void bwd_dkdv_kernel<64, true, true>(const KArgs);
+template __global__ void bwd_dkdv_kernel<128, false, false>(const KArgs);
+template __global__ void bwd_dkdv_kernel<128, false, true>(const KArgs);
+template __global__ void bwd_dkdv_kernel<128, true, false>(const KArgs);
+template __global__ void bwd_dkdv_kernel<128, true, true>(const KArgs);
 
 template <int D>
 static hipError_t launch_dq_d(const KArgs& a, bool ac, bool prod, int n_q_max, hipStream_t s) {

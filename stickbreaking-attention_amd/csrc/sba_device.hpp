@@ -168,7 +168,7 @@ __device__ __forceinline__ float prefix_sum32(float (&v)[16], int h, float base)
 //   carry  stick left after all visible keys NEWER than this sub-block:
 //          LOG space: log2 of it (<= 0);  PRODUCT space: the value itself.  Updated in place.
 //   p      out: weights A[q, key(i)]
-//   beta   out (NEED_BETA): sigmoid(z), 0 where masked
+//   beta   out (NEED_BETA): 1 - sigmoid(z) (the fraction of the stick a key leaves), 1 where masked
 //
 // Restates compute_block of the upstream Triton kernel
 // (stickbreaking_attention/sb_varlen/sb_varlen_fwd.py:26-78): base-2 softplus
@@ -199,7 +199,7 @@ __device__ __forceinline__ void stick_weights(const f32x16& x, float c, int k0, 
     for (int i = 1; i < 16; ++i) p[i] = ex[i] - ex[i - 1];
     if (NEED_BETA) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) beta[i] = 1.0f - r[i];
+      for (int i = 0; i < 16; ++i) beta[i] = r[i];
     }
   } else {
     float xs[16], sp[16];
@@ -209,8 +209,8 @@ __device__ __forceinline__ void stick_weights(const f32x16& x, float c, int k0, 
       xs[i] = fminf(c * x[i], 126.0f);
       const float t = 1.0f + fast_exp2(xs[i]);
       sp[i] = fast_log2(t);                  // base-2 softplus = -log2(1 - beta)
-      if (NEED_BETA) beta[i] = 1.0f - fast_rcp(t);
-      if (BAND && !(i < lim)) { sp[i] = 0.0f; if (NEED_BETA) beta[i] = 0.0f; }
+      if (NEED_BETA) beta[i] = fast_rcp(t);
+      if (BAND && !(i < lim)) { sp[i] = 0.0f; if (NEED_BETA) beta[i] = 1.0f; }
     }
     const float total = suffix_sum32(sp, h, -carry);
 #pragma unroll
@@ -304,30 +304,45 @@ __device__ __forceinline__ int swz_off(int row, int chunk) {   // element offset
 }
 
 // Asynchronous global -> LDS copy of ROWS x D bf16 of a (document, head) slice into an unpadded,
-// swizzled tile, issued by the THREADS threads whose index inside their group is `gtid`
-// (buffer_load_dwordx4 ... lds).  One wave instruction moves 1 KiB: lane l fills the 16-byte
-// LDS chunk number (first chunk of the instruction + l), so the swizzle (and the key
-// permutation of key tiles) is applied on the GLOBAL side by choosing which chunk a lane
-// fetches; rows past the end of the document arrive as zeros.  Completion is tracked by vmcnt:
-// wait for it, then barrier, before any wave reads the tile.
+// swizzled tile, issued by THREADS threads (buffer_load_dwordx4 ... lds).  One wave instruction
+// moves 1 KiB: lane l fills the 16-byte LDS chunk number (first chunk of the instruction + l),
+// so the swizzle (and the key permutation of key tiles) is applied on the GLOBAL side by
+// choosing which chunk a lane fetches; rows past the end of the document arrive as zeros.
+// Completion is tracked by vmcnt: wait for it, then barrier, before any wave reads the tile.
+// The per-lane part of the source offset is computed once (init); issuing a tile then costs
+// one add per instruction.
 template <int D, int ROWS, int THREADS, bool KEYS>
-__device__ __forceinline__ void async_tile(const Rows& r, int row0, unsigned short* lds_tile, int gtid) {
-  constexpr int C8 = D / 8;
-  constexpr int NCH = ROWS * C8 / THREADS;
+struct TileCopy {
+  static constexpr int C8 = D / 8;
+  static constexpr int NCH = ROWS * C8 / THREADS;
   static_assert(ROWS * C8 % THREADS == 0, "tile must split evenly over the loading threads");
-  const int wave = __builtin_amdgcn_readfirstlane(gtid >> 6), lane = gtid & 63;
+  int voff[NCH];   // byte offset of this lane's chunk relative to the tile's first row
+  int wave;
+
+  // gtid = index of the thread inside the group of THREADS loading threads
+  __device__ __forceinline__ void init(int gtid, unsigned row_bytes) {
+    wave = __builtin_amdgcn_readfirstlane(gtid >> 6);
+    const int lane = gtid & 63;
 #pragma unroll
-  for (int j = 0; j < NCH; ++j) {
-    const int chunk0 = (wave * NCH + j) * 64;       // wave-uniform
-    const int cidx = chunk0 + lane;
-    const int m = cidx / C8, phys = cidx % C8;
-    const int logical = phys ^ swz<D>(m);
-    const int src = KEYS ? ((m & ~31) | kperm(m & 31)) : m;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(
-        r.rsrc, (__attribute__((address_space(3))) void*)(lds_tile + chunk0 * 8), 16,
-        (row0 + src) * (int)r.row_bytes + logical * 16, 0, 0, 0);
+    for (int j = 0; j < NCH; ++j) {
+      const int cidx = (wave * NCH + j) * 64 + lane;
+      const int m = cidx / C8, phys = cidx % C8;
+      const int logical = phys ^ swz<D>(m);
+      const int src = KEYS ? ((m & ~31) | kperm(m & 31)) : m;
+      voff[j] = src * (int)row_bytes + logical * 16;
+    }
   }
-}
+
+  __device__ __forceinline__ void issue(const Rows& r, int row0, unsigned short* lds_tile) const {
+    const int base = __builtin_amdgcn_readfirstlane(row0 * (int)r.row_bytes);
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          r.rsrc, (__attribute__((address_space(3))) void*)(lds_tile + (wave * NCH + j) * 512), 16,
+          voff[j] + base, 0, 0, 0);
+    }
+  }
+};
 
 // Wait until at most N of this wave's global loads (including asynchronous tile copies) are
 // still in flight.

@@ -45,8 +45,11 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
 
   const int last_key = min(m0 + BM - 1, t.doc_len - 1);
   const int kt_last = last_key / BN;
-  async_tile<D, BN, NT, true>(krows, kt_last * BN, Ks, tid);
-  async_tile<D, BN, NT, true>(vrows, kt_last * BN, Vs, tid);
+  TileCopy<D, BN, NT, true> kcopy, vcopy;
+  kcopy.init(tid, krows.row_bytes);
+  vcopy.init(tid, vrows.row_bytes);
+  kcopy.issue(krows, kt_last * BN, Ks);
+  vcopy.issue(vrows, kt_last * BN, Vs);
 
   // Q^T operand fragments: lane (n, h) holds Q[qrow][16*ks + 8*h .. +7] (zeros past the document).
   bf16x8 qf[KS];
@@ -83,8 +86,8 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
     wait_loads<0>();
     lds_barrier();
     if (kt > 0) {
-      async_tile<D, BN, NT, true>(krows, (kt - 1) * BN, Ks + (buf ^ 1) * TILE, tid);
-      async_tile<D, BN, NT, true>(vrows, (kt - 1) * BN, Vs + (buf ^ 1) * TILE, tid);
+      kcopy.issue(krows, (kt - 1) * BN, Ks + (buf ^ 1) * TILE);
+      vcopy.issue(vrows, (kt - 1) * BN, Vs + (buf ^ 1) * TILE);
     }
     const unsigned short* Kt = Ks + buf * TILE;
     const unsigned short* Vt = Vs + buf * TILE;
@@ -143,6 +146,17 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
     }
   }
 }
+
+
+// Explicit instantiations: every (head_dim, attend_current, carry space) variant the launchers use.
+template __global__ void fwd_kernel<64, false, false>(const KArgs);
+template __global__ void fwd_kernel<64, false, true>(const KArgs);
+template __global__ void fwd_kernel<64, true, false>(const KArgs);
+template __global__ void fwd_kernel<64, true, true>(const KArgs);
+template __global__ void fwd_kernel<128, false, false>(const KArgs);
+template __global__ void fwd_kernel<128, false, true>(const KArgs);
+template __global__ void fwd_kernel<128, true, false>(const KArgs);
+template __global__ void fwd_kernel<128, true, true>(const KArgs);
 
 template <int D>
 static hipError_t launch_fwd_d(const KArgs& a, bool ac, bool prod, int n_q_max, hipStream_t s) {
