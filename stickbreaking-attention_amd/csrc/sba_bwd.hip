@@ -224,14 +224,8 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
     ce[1] = ce_next[1];
   }
 
-#pragma unroll
-  for (int db = 0; db < DB; ++db) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int row = qw0 + 8 * (i >> 2) + 4 * h + (i & 3);
-      if (row < t.doc_len) dqb[(int64_t)row * a.dq.st + 32 * db + n] = (__bf16)(dqacc[db][i] * a.inv_temp);
-    }
-  }
+  lds_barrier();   // every wave is done with the K/V tiles: their memory becomes the dq staging area
+  store_block32<D>(Ks + w * 32 * D, dqacc, a.inv_temp, dqb, a.dq.st, qw0, t.doc_len, lane);
 }
 
 // -------------------------------------------------------------------------------------------
@@ -254,20 +248,6 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
 constexpr int NT2 = 512;
 constexpr int BQ = 64;   // queries per step of the dk/dv pass
 
-// Experiment-only instrumentation (never defined in the shipped build): thread 0 of each role
-// accumulates shader-clock time per phase into the spare words of the schedule header.
-#ifdef SBA_PHASE_TIMING
-#define SBA_PH_DECL long long ph_t0 = clock64(); long long ph_acc[3] = {0, 0, 0};
-#define SBA_PH(i) { const long long ph_t1 = clock64(); ph_acc[i] += ph_t1 - ph_t0; ph_t0 = ph_t1; }
-#define SBA_PH_FLUSH(sched) if ((threadIdx.x & 255) == 0) { \
-    unsigned long long* d = reinterpret_cast<unsigned long long*>(const_cast<int*>(sched) + 4) + 3 * (threadIdx.x >> 8); \
-    for (int i = 0; i < 3; ++i) atomicAdd(d + i, (unsigned long long)ph_acc[i]); }
-#else
-#define SBA_PH_DECL
-#define SBA_PH(i)
-#define SBA_PH_FLUSH(sched)
-#endif
-
 template <int D, bool AC, bool PROD>
 __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   constexpr int KS = D / 16, DB = D / 32;
@@ -281,9 +261,6 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   __shared__ __attribute__((aligned(16))) unsigned short Ps[2 * PTILE];
   __shared__ __attribute__((aligned(16))) unsigned short Zs[2 * PTILE];
 
-#ifdef SBA_PHASE_TIMING
-  const long long wg_t0 = clock64();
-#endif
   const int* sched = a.sched;
   if (sched[SCHED_STATUS] != 0) return;
   const int slot = blockIdx.x / a.heads;
@@ -396,9 +373,6 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       settle(1, r1, ncarry_e, ncarry_c, ndr);
     }
     lds_barrier();                        // tiles 0 and 1 are in slots 0 and 1
-#ifdef SBA_PHASE_TIMING
-    const long long wg_t1 = clock64();
-#endif
     // One step: (xc, dc) hold the finished chains of block i; the chains of block i+1 go into
     // (xn, dn).  Called with the two accumulator pairs swapped on alternate steps, so nothing
     // is copied between steps.  FIRST = the step on the causal diagonal (masks, possible skip);
@@ -527,13 +501,6 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     }
     if (i < nsteps) later(i, xb, db, xa, da, rb, ra);
     lds_barrier();                        // the product waves' last step
-#ifdef SBA_PHASE_TIMING
-    if (threadIdx.x == 0) {
-      unsigned long long* d = reinterpret_cast<unsigned long long*>(const_cast<int*>(a.sched) + 4);
-      atomicAdd(d + 4, (unsigned long long)(wg_t1 - wg_t0));
-      atomicAdd(d + 5, (unsigned long long)(clock64() - wg_t0));
-    }
-#endif
   } else {
     __builtin_amdgcn_s_setprio(3);
     const int ptid = tid - NPT;
@@ -570,17 +537,9 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     fetch(1);
     wait_loads<0>();
     lds_barrier();
-    SBA_PH_DECL
     for (int i = 0; i <= nsteps; ++i) {
-#ifndef SBA_X_NO_STAGE
       if (i + 2 < nsteps) fetch(i + 2);
-#endif
-      SBA_PH(0)
-#ifdef SBA_X_NO_PRODUCTS
-      if (false) {
-#else
       if (i >= 1) {
-#endif
         // acc[key, d] += sum over the 64 queries of step i-1 of X[query][key] * Y[query][d]
         const unsigned short* Xt = (mat ? Zs : Ps) + ((i - 1) & 1) * PTILE;
         const unsigned short* Yt = (mat ? Qs : Gs) + ((i - 1) & 3) * QTILE;
@@ -603,26 +562,16 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
             for (int j = 0; j < DB; ++j) acc[j] = mfma32(af[k2], bf[k2][j], acc[j]);
         }
       }
-      SBA_PH(1)
       wait_loads<0>();   // tile i+2 has landed before anyone passes the barrier
       lds_barrier();
-      SBA_PH(2)
     }
-    SBA_PH_FLUSH(a.sched)
+    // (the last barrier of the loop has passed: the p/dz staging buffers are free)
     const View& ov = mat ? a.dk : a.dv;
     __bf16* outb = reinterpret_cast<__bf16*>(ov.ptr) + t.batch * ov.sb + head * ov.sh + tok0 * ov.st;
-    const float scale = mat ? a.inv_temp : 1.0f;
-#pragma unroll
-    for (int j = 0; j < DB; ++j) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int key = kt * BN + 32 * kb32 + 8 * (i >> 2) + 4 * h + (i & 3);
-        if (key < t.doc_len) outb[(int64_t)key * ov.st + 32 * j + n] = (__bf16)(acc[j][i] * scale);
-      }
-    }
+    unsigned short* scratch = (w & 2 ? Zs : Ps) + (w & 1) * 32 * D;
+    store_block32<D>(scratch, acc, mat ? a.inv_temp : 1.0f, outb, ov.st, kt * BN + 32 * kb32, t.doc_len, lane);
   }
 }
-
 
 // Explicit instantiations: every (head_dim, attend_current, carry space) variant the launchers use.
 template __global__ void bwd_dq_kernel<64, false, false>(const KArgs);

@@ -222,6 +222,91 @@ __device__ __forceinline__ void stick_weights(const f32x16& x, float c, int k0, 
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Epilogue: one wave writes its 32 x D block of fp32 accumulators (lane = column n of a 32-wide
+// block, register i = row 8*(i/4) + 4*h + i%4) to global memory as bf16.  Storing straight from
+// that layout would take 16*D/32 two-byte stores per lane; instead the block goes through a
+// wave-private LDS scratch of 32*D elements (2-byte LDS writes, 16-byte reads) and leaves as
+// D/16 fully coalesced 16-byte stores per lane.  Wave-private: no workgroup barrier inside,
+// but the caller must make sure nobody else still uses the scratch memory.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+__device__ __forceinline__ void store_block32(unsigned short* scratch, const f32x16 (&acc)[D / 32], float scale,
+                                              __bf16* out, int64_t stride_t, int row0, int limit, int lane) {
+  const int n = lane & 31, h = lane >> 5;
+  __bf16* sc = reinterpret_cast<__bf16*>(scratch);
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = 8 * (i >> 2) + 4 * h + (i & 3);
+      sc[row * D + 32 * db + n] = (__bf16)(acc[db][i] * scale);
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own LDS writes have landed
+  constexpr int C8 = D / 8;
+#pragma unroll
+  for (int j = 0; j < 32 * C8 / 64; ++j) {
+    const int cidx = lane + 64 * j;
+    const int row = cidx / C8, c8 = cidx % C8;
+    const uint4 v = *reinterpret_cast<const uint4*>(scratch + row * D + c8 * 8);
+    if (row0 + row < limit) *reinterpret_cast<uint4*>(out + (int64_t)(row0 + row) * stride_t + c8 * 8) = v;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same product-space arithmetic for an UNMASKED sub-block, cut into chunks with a caller
+// hook between them.  The hook is where a kernel issues MFMAs that do not depend on this
+// sub-block (the chains of the next one, the products of the previous one) and pins their
+// position with a scheduling barrier, so that the matrix core works underneath the VALU
+// stream instead of before or after it.
+//   weights_chunked:  hooks 0..3 after {r[0..7]}, {r[8..15]}, {stick chain}, {p}
+//   dz_chunked:       hooks 0..3 after {do.v - drem, totals}, {dz[0..7]}, {dz[8..15]}, {bf16 pack}
+// ---------------------------------------------------------------------------------------------
+template <class Hook>
+__device__ __forceinline__ void weights_chunked(const f32x16& x, float c, int h, float& carry,
+                                                float (&p)[16], float (&r)[16], Hook&& hook) {
+  float ex[16];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r[i] = fast_rcp(1.0f + fast_exp2(c * x[i]));
+  hook(0);
+#pragma unroll
+  for (int i = 8; i < 16; ++i) r[i] = fast_rcp(1.0f + fast_exp2(c * x[i]));
+  hook(1);
+  carry = suffix_prod32_excl(r, ex, h, carry);
+  hook(2);
+  p[0] = ex[0] - ex[0] * r[0];
+#pragma unroll
+  for (int i = 1; i < 16; ++i) p[i] = ex[i] - ex[i - 1];
+  hook(3);
+}
+
+template <class Hook>
+__device__ __forceinline__ void dz_chunked(const float (&p)[16], const float (&r)[16], const f32x16& da, int h,
+                                           float& carry_c, float dr, bf16x8 (&zf)[2], Hook&& hook) {
+  float dA[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) dA[i] = da[i] - dr;
+  float t0 = 0.0f, t1 = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 16; i += 2) { t0 = fmaf(p[i], dA[i], t0); t1 = fmaf(p[i + 1], dA[i + 1], t1); }
+  float lo, hi;
+  both_halves(t0 + t1, lo, hi);
+  float cprev = h == 1 ? carry_c + lo : carry_c;   // keys of the h=0 lane come first
+  hook(0);
+  float dz[16];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) { const float ci = fmaf(p[i], dA[i], cprev); dz[i] = fmaf(r[i], ci, -cprev); cprev = ci; }
+  hook(1);
+#pragma unroll
+  for (int i = 8; i < 16; ++i) { const float ci = fmaf(p[i], dA[i], cprev); dz[i] = fmaf(r[i], ci, -cprev); cprev = ci; }
+  hook(2);
+  carry_c += lo + hi;
+  zf[0] = pack8(dz);
+  zf[1] = pack8(dz + 8);
+  hook(3);
+}
+
 // Is the 32-key sub-block starting at k0 entirely invisible / entirely visible to the 32
 // queries starting at qw0?
 template <bool AC>

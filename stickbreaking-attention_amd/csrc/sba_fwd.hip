@@ -9,13 +9,16 @@
 namespace sba {
 
 template <int D, bool AC, bool PROD>
-__global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
+__global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   constexpr int KS = D / 16;     // contraction steps of K.Q^T
   constexpr int DB = D / 32;     // 32-wide output column blocks of P.V
-  constexpr int TILE = BN * D;   // elements of one K or V tile (unpadded, swizzled)
-  // K and V tiles, double-buffered, filled by asynchronous global -> LDS copies.
-  __shared__ __attribute__((aligned(16))) unsigned short Ks[2 * TILE];
-  __shared__ __attribute__((aligned(16))) unsigned short Vs[2 * TILE];
+  constexpr int BF = 32;         // keys per staged tile: one MFMA sub-block
+  constexpr int TILE = BF * D;   // elements of one K or V tile (unpadded, swizzled)
+  // K and V tiles of 32 keys, double-buffered, filled by asynchronous global -> LDS copies:
+  // 32 KiB per workgroup, so three workgroups share a CU.
+  __shared__ __attribute__((aligned(16))) unsigned short smem[4 * TILE];
+  unsigned short* const Ks = smem;              // two K tiles
+  unsigned short* const Vs = smem + 2 * TILE;   // two V tiles
 
   const int* sched = a.sched;
   if (sched[SCHED_STATUS] != 0) return;
@@ -44,12 +47,12 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
   const Rows vrows = make_rows(vb, a.v.st, t.doc_len);
 
   const int last_key = min(m0 + BM - 1, t.doc_len - 1);
-  const int kt_last = last_key / BN;
-  TileCopy<D, BN, NT, true> kcopy, vcopy;
+  const int kt_last = last_key / BF;
+  TileCopy<D, BF, NT, true> kcopy, vcopy;
   kcopy.init(tid, krows.row_bytes);
   vcopy.init(tid, vrows.row_bytes);
-  kcopy.issue(krows, kt_last * BN, Ks);
-  vcopy.issue(vrows, kt_last * BN, Vs);
+  kcopy.issue(krows, kt_last * BF, Ks);
+  vcopy.issue(vrows, kt_last * BF, Vs);
 
   // Q^T operand fragments: lane (n, h) holds Q[qrow][16*ks + 8*h .. +7] (zeros past the document).
   bf16x8 qf[KS];
@@ -86,17 +89,18 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
     wait_loads<0>();
     lds_barrier();
     if (kt > 0) {
-      kcopy.issue(krows, (kt - 1) * BN, Ks + (buf ^ 1) * TILE);
-      vcopy.issue(vrows, (kt - 1) * BN, Vs + (buf ^ 1) * TILE);
+      kcopy.issue(krows, (kt - 1) * BF, Ks + (buf ^ 1) * TILE);
+      vcopy.issue(vrows, (kt - 1) * BF, Vs + (buf ^ 1) * TILE);
     }
     const unsigned short* Kt = Ks + buf * TILE;
     const unsigned short* Vt = Vs + buf * TILE;
-#pragma unroll
-    for (int sb = 1; sb >= 0; --sb) {
-      const int k0 = kt * BN + 32 * sb;
+    buf ^= 1;
+    {
+      constexpr int sb = 0;
+      const int k0 = kt * BF;
       if (sub_skip<AC>(k0, qw0)) continue;
       // stick left on entering this sub-block: what both backward kernels start it from
-      if (stick != nullptr && h == 0 && qvalid) stick[(int64_t)(2 * kt + sb) * a.rows_total] = carry;
+      if (stick != nullptr && h == 0 && qvalid) stick[(int64_t)kt * a.rows_total] = carry;
       f32x16 x;
 #pragma unroll
       for (int i = 0; i < 16; ++i) x[i] = 0.0f;
@@ -129,7 +133,6 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
         for (int db = 0; db < DB; ++db) oacc[db] = mfma32(pf, vfr[tt][db], oacc[db]);
       }
     }
-    buf ^= 1;
   }
 
   // epilogue: rem = what is left of the stick; o rows in the accumulator layout
@@ -137,16 +140,9 @@ __global__ void __launch_bounds__(NT, 2) fwd_kernel(const KArgs a) {
     const float r = PROD ? carry : fast_exp2(carry);
     rb[(int64_t)qrow * a.rem.st] = (__bf16)r;
   }
-#pragma unroll
-  for (int db = 0; db < DB; ++db) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int row = qw0 + 8 * (i >> 2) + 4 * h + (i & 3);
-      if (row < t.doc_len) ob[(int64_t)row * a.o.st + 32 * db + n] = (__bf16)oacc[db][i];
-    }
-  }
+  lds_barrier();   // every wave is done with the K/V tiles: their memory becomes the o staging area
+  store_block32<D>(smem + w * 32 * D, oacc, 1.0f, ob, a.o.st, qw0, t.doc_len, lane);
 }
-
 
 // Explicit instantiations: every (head_dim, attend_current, carry space) variant the launchers use.
 template __global__ void fwd_kernel<64, false, false>(const KArgs);
