@@ -19,6 +19,13 @@ for p in (ROOT, os.path.join(ROOT, "stickbreaking-attention_amd")):
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X published dense bf16 MFMA peak
 
+# HBM bytes per launch on workload c3, from two `rocprofv3 --pmc` runs of this script
+# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, summed over XCDs), each scaled by what the
+# same counter reads for the 256 MiB device copy of --calibrate-copy (FETCH_SIZE x2.0,
+# WRITE_SIZE x1.0).  Counters cannot be read from inside the process, so these are recorded
+# constants; other workloads report null.
+MEASURED_TRAFFIC_BYTES = {"c3": {"fwd_kernel": 1.178e9, "bwd_dq_kernel": 1.071e9, "bwd_dkdv_kernel": 1.484e9}}
+
 
 def workload(name):
     with open(os.path.join(ROOT, "tests", "golden", "doc_lengths.json")) as f:
@@ -166,7 +173,9 @@ def main():
         "kernel_executed_tflops": {n: (executed[i] / (kern_ms[i] * 1e-3) / 1e12 if kern_ms[i] > 0 else 0.0)
                                    for i, n in enumerate(names)},
         "roofline": {"bound": "mfma", "kernel": names[dom], "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None},
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(names[dom])
+                     if _ops.PRODUCT_SPACE else None},
         "device": {"name": props.name, "cus": props.multi_processor_count,
                    "clock_mhz": getattr(props, "clock_rate", 0) / 1e3},
     }
