@@ -67,6 +67,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5"])
+    ap.add_argument("--lengths", default=None,
+                    help="comma-separated document lengths replacing the workload's own (shape sweeps; "
+                         "heads, head_dim and scaling stay those of --workload)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--log-space", action="store_true", help="log2-sum carry instead of product carry")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -85,6 +88,9 @@ def main():
     dev = torch.device("cuda:0")
     props = torch.cuda.get_device_properties(dev)
     lengths, cfg = workload(args.workload)
+    if args.lengths:
+        lengths = [int(x) for x in args.lengths.split(",")]
+        args.workload = f"{args.workload}/custom"
     H, d, T = cfg["H"], cfg["d"], sum(lengths)
     q, k, v, do = (t.to(dev) for t in orc.make_inputs((H, T, d), 1337, scale=cfg["scale"]))
     cu = torch.tensor(lengths, dtype=torch.int64).cumsum(0)

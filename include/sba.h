@@ -112,8 +112,9 @@ int sba_build_schedule(const sba_problem* p, void* schedule, void* stream);
 
 /* ---- forward ---------------------------------------------------------------------------- */
 
-/* o[b,h,t,:] and rem[b,h,t] for every token that belongs to a document; tokens outside any
- * document are left untouched (the caller zero-fills).  `stick_table` may be NULL when no
+/* o[b,h,t,:] and rem[b,h,t] for every token: tokens that belong to no document (past the
+ * last entry of cu_seqlens) are set to zero, as is everything when the scheduler rejected
+ * cu_seqlens.  `stick_table` may be NULL when no
  * backward will follow. */
 int sba_varlen_fwd(const sba_problem* p, const void* schedule,
                    const sba_view* q, const sba_view* k, const sba_view* v,
@@ -127,7 +128,7 @@ int sba_attn_fwd(const sba_problem* p, const void* schedule,
 
 /* ---- backward --------------------------------------------------------------------------- */
 
-/* dq, dk, dv for every token of every document (others untouched).  `stick_table` is the
+/* dq, dk, dv for every token (zero for tokens that belong to no document).  `stick_table` is the
  * table the forward filled for the same problem and inputs; `grad_table` is scratch of the
  * same size.  grad_rem may have ptr == NULL (treated as zeros). */
 int sba_varlen_bwd(const sba_problem* p, const void* schedule,

@@ -130,16 +130,25 @@ int forward(const sba_problem* p, bool fixed, const void* schedule, const sba_vi
   if ((e = check_mat(q, p)) || (e = check_mat(k, p)) || (e = check_mat(v, p)) || (e = check_mat(o, p))) return e;
   if ((e = check_view(rem, true))) return e;
   if ((e = check_arch())) return e;
-  if (sz.rows == 0 || sz.n_docs == 0) return 0;
+  if (sz.rows == 0) return 0;
   KArgs a;
   std::memset(&a, 0, sizeof(a));
   if ((e = fill_common(p, sz, schedule, &a))) return e;
   a.q = to_view(q); a.k = to_view(k); a.v = to_view(v); a.o = to_view(o); a.rem = to_view(rem);
   a.stick = stick;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  Timer tm(0, s);
-  return (int)launch_fwd(a, p->head_dim, (p->flags & SBA_ATTEND_CURRENT) != 0,
-                         (p->flags & SBA_PRODUCT_SPACE) != 0, sz.n_q_max, s);
+  hipError_t he = hipSuccess;
+  if (sz.n_docs > 0) {
+    Timer tm(0, s);
+    he = launch_fwd(a, p->head_dim, (p->flags & SBA_ATTEND_CURRENT) != 0,
+                    (p->flags & SBA_PRODUCT_SPACE) != 0, sz.n_q_max, s);
+  }
+  if (he != hipSuccess || fixed) return (int)he;
+  ZeroArgs z;
+  std::memset(&z, 0, sizeof(z));
+  z.mat[0] = a.o; z.n_mat = 1; z.row = a.rem;
+  z.sched = a.sched; z.heads = p->heads; z.tokens = p->tokens; z.head_dim = p->head_dim;
+  return (int)launch_zero_tail(z, s);
 }
 
 int backward(const sba_problem* p, bool fixed, const void* schedule, const sba_view* q, const sba_view* k,
@@ -153,7 +162,7 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, const sba_v
     return e;
   if (stick == nullptr || gtab == nullptr) return SBA_E_NULL;
   if ((e = check_arch())) return e;
-  if (sz.rows == 0 || sz.n_docs == 0) return 0;
+  if (sz.rows == 0) return 0;
   KArgs a;
   std::memset(&a, 0, sizeof(a));
   if ((e = fill_common(p, sz, schedule, &a))) return e;
@@ -164,17 +173,24 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, const sba_v
   a.gtab = gtab;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const bool ac = (p->flags & SBA_ATTEND_CURRENT) != 0, prod = (p->flags & SBA_PRODUCT_SPACE) != 0;
-  hipError_t he;
-  {
-    Timer tm(1, s);
-    he = launch_bwd_dq(a, p->head_dim, ac, prod, sz.n_q_max, s);
+  hipError_t he = hipSuccess;
+  if (sz.n_docs > 0) {
+    {
+      Timer tm(1, s);
+      he = launch_bwd_dq(a, p->head_dim, ac, prod, sz.n_q_max, s);
+    }
+    if (he != hipSuccess) return (int)he;
+    {
+      Timer tm(2, s);
+      he = launch_bwd_dkdv(a, p->head_dim, ac, prod, sz.n_kv_max, s);
+    }
   }
-  if (he != hipSuccess) return (int)he;
-  {
-    Timer tm(2, s);
-    he = launch_bwd_dkdv(a, p->head_dim, ac, prod, sz.n_kv_max, s);
-  }
-  return (int)he;
+  if (he != hipSuccess || fixed) return (int)he;
+  ZeroArgs z;
+  std::memset(&z, 0, sizeof(z));
+  z.mat[0] = a.dq; z.mat[1] = a.dk; z.mat[2] = a.dv; z.n_mat = 3;
+  z.sched = a.sched; z.heads = p->heads; z.tokens = p->tokens; z.head_dim = p->head_dim;
+  return (int)launch_zero_tail(z, s);
 }
 
 }  // namespace

@@ -31,6 +31,7 @@ constexpr int SCHED_STATUS = 0;
 constexpr int SCHED_NQ = 1;      // number of query tiles
 constexpr int SCHED_NKV = 2;     // number of KV tiles
 constexpr int SCHED_MAXLEN = 3;  // longest document found
+constexpr int SCHED_TOTAL = 4;   // tokens covered by the documents (0 when the input is rejected)
 constexpr int SCHED_HDR = 16;    // tile lists start here
 
 struct Tile {

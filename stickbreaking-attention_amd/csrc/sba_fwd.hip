@@ -1,10 +1,12 @@
 // Forward kernel: one 128-row query tile of one (document, head) per workgroup, KV tiles of
-// 64 keys walked from the causal diagonal back to the start of the document.
+// 32 keys walked from the causal diagonal back to the start of the document.
 //
 // Replaces upstream `_forward` / `_forward_one_row`
 // (stickbreaking_attention/sb_varlen/sb_varlen_fwd.py:81-215, :231-410) and the fixed-length
 // wrapper (stickbreaking_attention/sb_attn/sb_fwd.py:15-136).
 #include "sba_kernels.hpp"
+
+#include <type_traits>
 
 namespace sba {
 
@@ -14,11 +16,11 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   constexpr int DB = D / 32;     // 32-wide output column blocks of P.V
   constexpr int BF = 32;         // keys per staged tile: one MFMA sub-block
   constexpr int TILE = BF * D;   // elements of one K or V tile (unpadded, swizzled)
-  // K and V tiles of 32 keys, double-buffered, filled by asynchronous global -> LDS copies:
-  // 32 KiB per workgroup, so three workgroups share a CU.
-  __shared__ __attribute__((aligned(16))) unsigned short smem[4 * TILE];
-  unsigned short* const Ks = smem;              // two K tiles
-  unsigned short* const Vs = smem + 2 * TILE;   // two V tiles
+  // K and V tiles of 32 keys in a three-slot ring filled by asynchronous global -> LDS copies:
+  // 48 KiB per workgroup, so three workgroups share a CU.
+  __shared__ __attribute__((aligned(16))) unsigned short smem[6 * TILE];
+  unsigned short* const Ks = smem;              // three K tiles
+  unsigned short* const Vs = smem + 3 * TILE;   // three V tiles
 
   const int* sched = a.sched;
   if (sched[SCHED_STATUS] != 0) return;
@@ -48,16 +50,23 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
 
   const int last_key = min(m0 + BM - 1, t.doc_len - 1);
   const int kt_last = last_key / BF;
-  TileCopy<D, BF, NT, true> kcopy, vcopy;
-  kcopy.init(tid, krows.row_bytes);
-  vcopy.init(tid, vrows.row_bytes);
-  kcopy.issue(krows, kt_last * BF, Ks);
-  vcopy.issue(vrows, kt_last * BF, Vs);
 
   // Q^T operand fragments: lane (n, h) holds Q[qrow][16*ks + 8*h .. +7] (zeros past the document).
   bf16x8 qf[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) qf[ks] = load_frag(qrows, qrow, 32 * ks + 16 * h);
+
+  // Three-stage ring of K/V tiles: two tiles are in flight while one is consumed.
+  TileCopy<D, BF, NT, true> kcopy, vcopy;
+  kcopy.init(tid, krows.row_bytes);
+  vcopy.init(tid, vrows.row_bytes);
+  constexpr int LOADS_PER_TILE = 2 * TileCopy<D, BF, NT, true>::NCH;
+  kcopy.issue(krows, kt_last * BF, Ks);
+  vcopy.issue(vrows, kt_last * BF, Vs);
+  if (kt_last >= 1) {
+    kcopy.issue(krows, (kt_last - 1) * BF, Ks + TILE);
+    vcopy.issue(vrows, (kt_last - 1) * BF, Vs + TILE);
+  }
 
   f32x16 oacc[DB];
 #pragma unroll
@@ -67,7 +76,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   float carry = PROD ? 1.0f : 0.0f;
 
   // Offsets (elements) inside a tile.  K: row read of chunk 2*ks + h of LDS row n (= MFMA row n).
-  // V: transpose reads of rows 8*u + 4*h + i/4 (+ 32*sb + 16*tt), columns 32*db + 16*blk + 4*(i%4).
+  // V: transpose reads of rows 8*u + 4*h + i/4 (+ 16*tt), columns 32*db + 16*blk + 4*(i%4).
   const int i16 = lane & 15, blk = (lane >> 4) & 1;
   int koff[KS], voff[2][DB];
 #pragma unroll
@@ -83,56 +92,65 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   }
   float* stick = a.stick == nullptr ? nullptr : a.stick + (int64_t)head * a.n_tt * a.rows_total + grow;
 
-  int buf = 0;
-  for (int kt = kt_last; kt >= 0; --kt) {
-    // tile kt has landed and every wave is done with the tile before it
-    wait_loads<0>();
+  // One tile step; the ring slot is a compile-time constant so every LDS address is a fixed
+  // register plus an immediate.
+  auto tile = [&](auto slot_c, const int kt) {
+    constexpr int SLOT = decltype(slot_c)::value;
+    constexpr int REFILL = (SLOT + 2) % 3;   // slot of tile kt + 1, free once every wave is past it
+    // Tile kt has landed when only the loads of tile kt - 1 (issued after it, returning in
+    // order) can still be in flight; stores in between only make the wait stricter.
+    if (kt >= 1) wait_loads<LOADS_PER_TILE>(); else wait_loads<0>();
     lds_barrier();
-    if (kt > 0) {
-      kcopy.issue(krows, (kt - 1) * BF, Ks + (buf ^ 1) * TILE);
-      vcopy.issue(vrows, (kt - 1) * BF, Vs + (buf ^ 1) * TILE);
+    if (kt >= 2) {
+      kcopy.issue(krows, (kt - 2) * BF, Ks + REFILL * TILE);
+      vcopy.issue(vrows, (kt - 2) * BF, Vs + REFILL * TILE);
     }
-    const unsigned short* Kt = Ks + buf * TILE;
-    const unsigned short* Vt = Vs + buf * TILE;
-    buf ^= 1;
+    const unsigned short* Kt = Ks + SLOT * TILE;
+    const unsigned short* Vt = Vs + SLOT * TILE;
+    const int k0 = kt * BF;
+    if (sub_skip<AC>(k0, qw0)) return;
+    // stick left on entering this block: what both backward kernels start it from
+    if (stick != nullptr && h == 0 && qvalid) stick[(int64_t)kt * a.rows_total] = carry;
+    f32x16 x;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) x[i] = 0.0f;
     {
-      constexpr int sb = 0;
-      const int k0 = kt * BF;
-      if (sub_skip<AC>(k0, qw0)) continue;
-      // stick left on entering this sub-block: what both backward kernels start it from
-      if (stick != nullptr && h == 0 && qvalid) stick[(int64_t)kt * a.rows_total] = carry;
-      f32x16 x;
+      bf16x8 kfr[KS];
 #pragma unroll
-      for (int i = 0; i < 16; ++i) x[i] = 0.0f;
-      {
-        bf16x8 kfr[KS];
+      for (int ks = 0; ks < KS; ++ks) kfr[ks] = lds_row8(Kt + koff[ks]);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) kfr[ks] = lds_row8(Kt + 32 * sb * D + koff[ks]);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) x = mfma32(kfr[ks], qf[ks], x);
-      }
-      float p[16], unused[16];
-      if (sub_full<AC>(k0, qw0)) {
-        stick_weights<AC, PROD, false, false>(x, a.c, k0, qrow, h, carry, p, unused);
-      } else {
-        stick_weights<AC, PROD, true, false>(x, a.c, k0, qrow, h, carry, p, unused);
-      }
-      // P as the A operand of O = P.V: slot s of step tt is key 16*h + 8*tt + s, which the
-      // permuted tile keeps in LDS row 16*tt + 8*(s/4) + 4*h + s%4.
-      bf16x8 vfr[2][DB];
-#pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-        const unsigned short* vrow = Vt + (32 * sb + 16 * tt) * D;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) vfr[tt][db] = lds_tr8(vrow + voff[0][db], vrow + voff[1][db]);
-      }
-#pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-        const bf16x8 pf = pack8(p + 8 * tt);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) oacc[db] = mfma32(pf, vfr[tt][db], oacc[db]);
-      }
+      for (int ks = 0; ks < KS; ++ks) x = mfma32(kfr[ks], qf[ks], x);
     }
+    float p[16], unused[16];
+    if (sub_full<AC>(k0, qw0)) {
+      stick_weights<AC, PROD, false, false>(x, a.c, k0, qrow, h, carry, p, unused);
+    } else {
+      stick_weights<AC, PROD, true, false>(x, a.c, k0, qrow, h, carry, p, unused);
+    }
+    // P as the A operand of O = P.V: slot s of step tt is key 16*h + 8*tt + s, which the
+    // permuted tile keeps in LDS row 16*tt + 8*(s/4) + 4*h + s%4.
+    bf16x8 vfr[2][DB];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      const unsigned short* vrow = Vt + 16 * tt * D;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) vfr[tt][db] = lds_tr8(vrow + voff[0][db], vrow + voff[1][db]);
+    }
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      const bf16x8 pf = pack8(p + 8 * tt);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) oacc[db] = mfma32(pf, vfr[tt][db], oacc[db]);
+    }
+  };
+
+  for (int kt = kt_last;;) {
+    tile(std::integral_constant<int, 0>{}, kt);
+    if (--kt < 0) break;
+    tile(std::integral_constant<int, 1>{}, kt);
+    if (--kt < 0) break;
+    tile(std::integral_constant<int, 2>{}, kt);
+    if (--kt < 0) break;
   }
 
   // epilogue: rem = what is left of the stick; o rows in the accumulator layout

@@ -32,7 +32,17 @@ struct SchedArgs {
   int* out;
 };
 
+// Rows of packed variable-length outputs that belong to no document.
+struct ZeroArgs {
+  View mat[3];      // [heads, tokens, head_dim] outputs to clear past the last document
+  int n_mat;
+  View row;         // per-row output (rem); ptr may be null
+  const int* sched;
+  int heads, tokens, head_dim;
+};
+
 hipError_t launch_schedule(const SchedArgs& a, hipStream_t s);
+hipError_t launch_zero_tail(const ZeroArgs& a, hipStream_t s);
 hipError_t launch_fwd(const KArgs& a, int head_dim, bool attend_current, bool product, int n_q_max,
                       hipStream_t s);
 hipError_t launch_bwd_dq(const KArgs& a, int head_dim, bool attend_current, bool product, int n_q_max,

@@ -112,9 +112,10 @@ def forward(plan: Plan, q, k, v, need_table: bool) -> Tuple[torch.Tensor, torch.
     fixed = plan.fixed
     qp, kp, vp = (_prep(t, plan.head_dim) for t in (q, k, v))
     padded = plan.head_dim != plan.orig_head_dim or q.dtype != torch.bfloat16
-    # Tokens outside every document are defined as zero (upstream leaves them uninitialised).
-    o = torch.zeros_like(qp) if not fixed else torch.empty_like(qp)
-    rem = torch.zeros_like(qp[..., 0])
+    # Every row is written by the library: rows of documents by the forward kernel, rows that
+    # belong to no document are cleared (upstream leaves those uninitialised).
+    o = torch.empty_like(qp)
+    rem = torch.empty_like(qp[..., 0])
     table = None
     if need_table:
         table = torch.empty(plan.table_bytes // 4, dtype=torch.float32, device=q.device)
@@ -142,8 +143,7 @@ def backward(plan: Plan, q, k, v, do, drem, table, dkdv_dtype=None):
     if drem is not None:
         dremp = drem if drem.dtype == torch.bfloat16 else drem.to(torch.bfloat16)
     padded = plan.head_dim != plan.orig_head_dim or q.dtype != torch.bfloat16
-    zeros = torch.empty_like if fixed else torch.zeros_like
-    dq, dk, dv = zeros(qp), zeros(kp), zeros(vp)
+    dq, dk, dv = torch.empty_like(qp), torch.empty_like(kp), torch.empty_like(vp)
     gtab = torch.empty(plan.table_bytes // 4, dtype=torch.float32, device=q.device)
     fn = lib.sba_attn_bwd if fixed else lib.sba_varlen_bwd
     with torch.cuda.device(q.device):

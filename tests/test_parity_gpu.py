@@ -90,11 +90,41 @@ def test_ragged_documents(lengths, ac, d):
     check_all(run_varlen(q, k, v, do, lengths, ac, drem=drem), oracle_varlen(q, k, v, do, lengths, ac, drem=drem))
 
 
+def _poison_free_blocks(shape, n=6):
+    # The operators allocate their outputs uninitialised; leave NaN patterns in the allocator's
+    # free blocks of that size so that a row nobody writes cannot pass for a zero.
+    blocks = [torch.full(shape, float("nan"), dtype=torch.bfloat16, device=DEV) for _ in range(n)]
+    blocks += [torch.full(shape[:-1], float("nan"), dtype=torch.bfloat16, device=DEV) for _ in range(n)]
+    torch.cuda.synchronize()
+    del blocks
+
+
+def test_rejected_cu_seqlens_give_zero_outputs():
+    from stickbreaking_attention import sb_attn_varlen
+    q = torch.randn(2, 256, 64, device=DEV).to(torch.bfloat16)
+    _poison_free_blocks((2, 256, 64))
+    with torch.no_grad():
+        o, rem = sb_attn_varlen(q, q, q, torch.tensor([100, 50, 256], dtype=torch.int32, device=DEV), 256, zero_start=False)
+    torch.cuda.synchronize()
+    assert (o == 0).all() and (rem == 0).all()
+
+
+def test_no_documents_give_zero_outputs():
+    from stickbreaking_attention import sb_attn_varlen
+    q = torch.randn(2, 128, 64, device=DEV).to(torch.bfloat16).requires_grad_()
+    _poison_free_blocks((2, 128, 64))
+    o, rem = sb_attn_varlen(q, q, q, torch.zeros(0, dtype=torch.int32, device=DEV), 128, zero_start=False)
+    (dq,) = torch.autograd.grad(o, (q,), torch.ones_like(o))
+    torch.cuda.synchronize()
+    assert (o == 0).all() and (rem == 0).all() and (dq == 0).all()
+
+
 def test_empty_documents_and_tail_tokens():
     # zero-length documents in the middle, and 40 tokens after the last document
     lengths = [50, 0, 0, 130, 0, 20]
     T = sum(lengths) + 40
     q, k, v, do = orc.make_inputs((2, T, 64), 11)
+    _poison_free_blocks((2, T, 64))
     got = run_varlen(q, k, v, do, lengths)
     ref = oracle_varlen(q, k, v, do, lengths)
     check_all(got, ref)
