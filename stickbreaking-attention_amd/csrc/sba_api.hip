@@ -39,7 +39,7 @@ int check_problem(const sba_problem* p, bool fixed, Sizes* sz) {
   sz->n_docs = fixed ? p->batch : p->n_docs;
   sz->rows = (long long)p->batch * p->tokens;
   sz->n_q_max = (int)(sz->rows / BM) + sz->n_docs + 1;
-  sz->n_kv_max = (int)(sz->rows / BN) + sz->n_docs + 1;
+  sz->n_kv_max = (int)(sz->rows / BKV) + sz->n_docs + 1;
   sz->n_tt = cdiv_i(p->max_doc_len > 0 ? p->max_doc_len : 1, BT);
   return 0;
 }

@@ -229,34 +229,35 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
 }
 
 // -------------------------------------------------------------------------------------------
-// dk / dv pass.  One workgroup owns 64 keys of one (document, head) and walks the queries that
-// can see them, 64 at a time.  Its 8 waves are specialised so that every SIMD hosts one
-// VALU-bound and one MFMA-bound wave that run concurrently:
+// dk / dv pass.  One workgroup owns 128 keys of one (document, head) and walks the queries that
+// can see them, 32 at a time.  Its 8 waves are specialised:
 //
-//   waves 0-3  "score" waves (query group qg, key sub-block sb): recompute the 32x32 block of
-//              p and dz of step i (K and V fragments live in registers) and stage them in LDS.
+//   waves 0-3  "score" waves, one 32-key block each: recompute the 32x32 block of p and dz of
+//              step i (K and V fragments live in registers) and stage them in LDS.
 //              Software-pipelined: the two MFMA chains (q.k and do.v) of block i+1 are issued
 //              while the VALU works on block i.
 //   waves 4-7  "product" waves: accumulate dv = p^T dO and dk = dz^T Q of step i-1 from the
-//              staged blocks (each owns 32 keys x D of one of the two outputs), and do all the
-//              global -> LDS staging of the Q/dO tiles, two steps ahead.
+//              staged blocks (each owns 64 keys x D of one of the two outputs), and do all the
+//              global -> LDS staging of the Q/dO tiles, four steps ahead.
 //
-// p/dz staging is double-buffered and the Q/dO tiles sit in a ring of four slots (in step i:
-// slot i-1 feeds the products, slot i+1 the score chains, slot i+2 is being filled), so a step
-// needs a single workgroup barrier.
+// p/dz staging is double-buffered and the Q/dO tiles sit in a ring of eight slots (in step i:
+// slot i-1 feeds the products, slot i+1 the score chains, slots i+2..i+4 are in flight), so a
+// step needs a single workgroup barrier and a tile has three steps to arrive.
 // -------------------------------------------------------------------------------------------
 constexpr int NT2 = 512;
-constexpr int BQ = 64;   // queries per step of the dk/dv pass
+constexpr int BQ = 32;     // queries per step of the dk/dv pass
+constexpr int RING = 8;    // Q/dO tile slots
+constexpr int AHEAD = 4;   // a tile is requested this many steps before the products use it + 1
 
 template <int D, bool AC, bool PROD>
 __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   constexpr int KS = D / 16, DB = D / 32;
   constexpr int NPT = NT2 / 2;                 // threads of one role
-  constexpr int QTILE = BQ * D;    // elements of one Q or dO tile (swizzled, unpadded)
-  constexpr int PTILE = BQ * BN;   // elements of one staged p or dz block [query][key]
+  constexpr int QTILE = BQ * D;     // elements of one Q or dO tile (swizzled, unpadded)
+  constexpr int PTILE = BQ * BKV;   // elements of one staged p or dz block [query][key]
   // Q and dO tiles: row reads (score operands) and transpose reads (dk/dv operands).
-  __shared__ __attribute__((aligned(16))) unsigned short Qs[4 * QTILE];
-  __shared__ __attribute__((aligned(16))) unsigned short Gs[4 * QTILE];
+  __shared__ __attribute__((aligned(16))) unsigned short Qs[RING * QTILE];
+  __shared__ __attribute__((aligned(16))) unsigned short Gs[RING * QTILE];
   // p and dz staged [query][key]: 16-byte row writes, transpose reads.
   __shared__ __attribute__((aligned(16))) unsigned short Ps[2 * PTILE];
   __shared__ __attribute__((aligned(16))) unsigned short Zs[2 * PTILE];
@@ -287,7 +288,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   const Rows krows = make_rows(kb, a.k.st, t.doc_len);
   const Rows vrows = make_rows(vb, a.v.st, t.doc_len);
 
-  const int q_first = kt * BN;                                   // first query that can see the tile
+  const int q_first = kt * BKV;                                  // first query that can see the tile
   const int nsteps = (t.doc_len - q_first + BQ - 1) / BQ;        // >= 1
 
   // The two roles run separate copies of the step loop (same barrier count) so that neither
@@ -297,17 +298,21 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   // waves, whose long VALU streams would otherwise starve them and serialise the two roles.
   if (scorer) {
     __builtin_amdgcn_s_setprio(0);
-    const int qg = (w >> 1) & 1, sb = w & 1;
-    const int k0 = kt * BN + 32 * sb;
-    const int qr = 32 * qg + n;                 // this lane's query row inside a tile
+    const int sb = w;                           // 32-key block of this wave
+    const int k0 = kt * BKV + 32 * sb;
+    const int qr = n;                           // this lane's query row inside a tile
     bf16x8 kf[KS], vf[KS];                      // MFMA row n holds key k0 + kperm(n)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       kf[ks] = load_frag(krows, k0 + kperm(n), 32 * ks + 16 * h);
       vf[ks] = load_frag(vrows, k0 + kperm(n), 32 * ks + 16 * h);
     }
+    // A block that starts past the end of the document is never visible to a query; its table
+    // reads are redirected to the document's last block so that they stay inside the tables
+    // (which hold ceil(max_doc_len / 32) blocks per row), and their values are never used.
+    const int tblock = min((BKV / 32) * kt + sb, (t.doc_len - 1) / 32);
     const int64_t tab = (int64_t)head * a.n_tt * a.rows_total + (int64_t)t.batch * a.tokens + tok0 +
-                        (int64_t)(2 * kt + sb) * a.rows_total;
+                        (int64_t)tblock * a.rows_total;
     // Per-row carries of a step, branch-free: the address is clamped into the document and the
     // value replaced by the neutral element past its end (those rows have zero Q and dO).
     const int64_t grem_st = grb != nullptr ? a.grem.st : 0;
@@ -333,9 +338,9 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     int roff[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) roff[ks] = swz_off<D>(qr, 2 * ks + h);
-    auto chains = [&](int slot4, f32x16& x, f32x16& da) {
-      const unsigned short* Qt = Qs + slot4 * QTILE;
-      const unsigned short* Gt = Gs + slot4 * QTILE;
+    auto chains = [&](int slot8, f32x16& x, f32x16& da) {
+      const unsigned short* Qt = Qs + slot8 * QTILE;
+      const unsigned short* Gt = Gs + slot8 * QTILE;
 #pragma unroll
       for (int j = 0; j < 16; ++j) { x[j] = 0.0f; da[j] = 0.0f; }
       // all operand reads first, so the chains are not paced by LDS latency
@@ -355,8 +360,8 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt) {
         const int chunk = 4 * sb + 2 * h + tt;
-        *reinterpret_cast<bf16x8*>(Pt + swz_off<BN>(qr, chunk)) = pf[tt];
-        *reinterpret_cast<bf16x8*>(Zt + swz_off<BN>(qr, chunk)) = zf[tt];
+        *reinterpret_cast<bf16x8*>(Pt + swz_off<BKV>(qr, chunk)) = pf[tt];
+        *reinterpret_cast<bf16x8*>(Zt + swz_off<BKV>(qr, chunk)) = zf[tt];
       }
     };
 
@@ -375,22 +380,22 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     lds_barrier();                        // tiles 0 and 1 are in slots 0 and 1
     // One step: (xc, dc) hold the finished chains of block i; the chains of block i+1 go into
     // (xn, dn).  Called with the two accumulator pairs swapped on alternate steps, so nothing
-    // is copied between steps.  FIRST = the step on the causal diagonal (masks, possible skip);
-    // every later step is one straight-line block in which the MFMA chains of block i+1 are
-    // interleaved with the VALU work on block i.
-    auto step = [&](auto first_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& req,
+    // is copied between steps.  DIAG = one of the first steps, whose queries may sit on or
+    // above this wave's keys (masks, possible skip); every later step is one straight-line
+    // block in which the MFMA chains of block i+1 are interleaved with the VALU work on block i.
+    auto step = [&](auto diag_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& req,
                     const Raw& due) {
-      constexpr bool FIRST = decltype(first_tag)::value;
+      constexpr bool DIAG = decltype(diag_tag)::value;
       request(i + 3, req);
-      chains((i + 1) & 3, xn, dn);
+      chains((i + 1) & (RING - 1), xn, dn);
       bf16x8 pf[2], zf[2];
-      const int qw0 = q_first + i * BQ + 32 * qg;
+      const int qw0 = q_first + i * BQ;
       const int qrow = qw0 + n;
-      if (FIRST && sub_skip<AC>(k0, qw0)) {
+      if (DIAG && sub_skip<AC>(k0, qw0)) {
         pf[0] = zero8(); pf[1] = zero8(); zf[0] = zero8(); zf[1] = zero8();
       } else {
         float p[16], bt[16];
-        if (FIRST) grad_weights<AC, PROD>(xc, a.c, k0, qw0, qrow, h, carry_e, p, bt);
+        if (DIAG) grad_weights<AC, PROD>(xc, a.c, k0, qw0, qrow, h, carry_e, p, bt);
         else stick_weights<AC, PROD, false, true>(xc, a.c, k0, qrow, h, carry_e, p, bt);
         pf[0] = pack8(p);
         pf[1] = pack8(p + 8);
@@ -404,48 +409,54 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     };
     // The same step for the product-space carry away from the diagonal, hand-pipelined: the
     // VALU work on block i is cut into 8 chunks and the 2*KS chain MFMAs of block i+1 are
-    // issued between them (operand reads one chunk ahead), each position pinned with a
+    // issued between them (operand reads two chunks ahead), each position pinned with a
     // scheduling barrier so that the matrix core runs underneath the VALU stream.
     auto bulk = [&](int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& req, const Raw& due) {
       constexpr int NCHUNK = 8, PER = 2 * KS / NCHUNK;
       request(i + 3, req);
-      const unsigned short* Qt = Qs + ((i + 1) & 3) * QTILE;
-      const unsigned short* Gt = Gs + ((i + 1) & 3) * QTILE;
+      const unsigned short* Qt = Qs + ((i + 1) & (RING - 1)) * QTILE;
+      const unsigned short* Gt = Gs + ((i + 1) & (RING - 1)) * QTILE;
 #pragma unroll
       for (int j = 0; j < 16; ++j) { xn[j] = 0.0f; dn[j] = 0.0f; }
-      bf16x8 fr[PER];
+      // Operand reads run LEAD chunks ahead of the MFMAs that consume them (LDS latency under
+      // load is longer than one chunk of VALU work), through a small rotating set of registers.
+      constexpr int LEAD = 2;
+      bf16x8 fr[LEAD + 1][PER];
       auto pre = [&](int c) {
+        if (c >= NCHUNK) return;
 #pragma unroll
         for (int m = 0; m < PER; ++m) {
           const int k = c * PER + m;   // even: q.k chain step k/2, odd: do.v chain step k/2
-          fr[m] = lds_row8(((k & 1) ? Gt : Qt) + roff[k >> 1]);
+          fr[c % (LEAD + 1)][m] = lds_row8(((k & 1) ? Gt : Qt) + roff[k >> 1]);
         }
       };
       auto post = [&](int c) {
 #pragma unroll
         for (int m = 0; m < PER; ++m) {
           const int k = c * PER + m;
-          if (k & 1) dn = mfma32(vf[k >> 1], fr[m], dn);
-          else xn = mfma32(kf[k >> 1], fr[m], xn);
+          if (k & 1) dn = mfma32(vf[k >> 1], fr[c % (LEAD + 1)][m], dn);
+          else xn = mfma32(kf[k >> 1], fr[c % (LEAD + 1)][m], xn);
         }
         __builtin_amdgcn_sched_barrier(0);
       };
+      pre(0);
+      pre(1);
       float r[16], ex[16], p[16];
       // chunks 0, 1: r = 1 - beta of the 16 keys
-      pre(0);
+      pre(2);
 #pragma unroll
       for (int j = 0; j < 8; ++j) r[j] = fast_rcp(1.0f + fast_exp2(a.c * xc[j]));
       post(0);
-      pre(1);
+      pre(3);
 #pragma unroll
       for (int j = 8; j < 16; ++j) r[j] = fast_rcp(1.0f + fast_exp2(a.c * xc[j]));
       post(1);
       // chunk 2: stick left after the newer keys
-      pre(2);
+      pre(4);
       carry_e = suffix_prod32_excl(r, ex, h, carry_e);
       post(2);
       // chunk 3: weights and their bf16 fragments
-      pre(3);
+      pre(5);
       p[0] = ex[0] - ex[0] * r[0];
 #pragma unroll
       for (int j = 1; j < 16; ++j) p[j] = ex[j] - ex[j - 1];
@@ -454,7 +465,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       pf[1] = pack8(p + 8);
       post(3);
       // chunk 4: do.v - drem and this lane's total of G
-      pre(4);
+      pre(6);
       float dA[16];
 #pragma unroll
       for (int j = 0; j < 16; ++j) dA[j] = dc[j] - dr;
@@ -467,16 +478,16 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       post(4);
       // chunks 5, 6: running sum of G and dz = r C[i] - C[i-1]
       float dz[16];
-      pre(5);
+      pre(7);
 #pragma unroll
       for (int j = 0; j < 8; ++j) { const float cj = fmaf(p[j], dA[j], cprev); dz[j] = fmaf(r[j], cj, -cprev); cprev = cj; }
       post(5);
-      pre(6);
+      pre(8);
 #pragma unroll
       for (int j = 8; j < 16; ++j) { const float cj = fmaf(p[j], dA[j], cprev); dz[j] = fmaf(r[j], cj, -cprev); cprev = cj; }
       post(6);
       // chunk 7: dz fragments and staging
-      pre(7);
+      pre(9);
       zf[0] = pack8(dz);
       zf[1] = pack8(dz + 8);
       stage(i, pf, zf);
@@ -493,31 +504,42 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     };
     f32x16 xa, da, xb, db;
     chains(0, xa, da);
-    step(std::true_type{}, 0, xa, da, xb, db, ra, rb);
-    int i = 1;
-    for (; i + 1 < nsteps; i += 2) {
-      later(i, xb, db, xa, da, rb, ra);
-      later(i + 1, xa, da, xb, db, ra, rb);
+    // the first BKV/BQ steps can touch the diagonal of some wave's block
+    int i = 0;
+#pragma unroll 1
+    for (; i < BKV / BQ && i < nsteps; i += 2) {
+      step(std::true_type{}, i, xa, da, xb, db, ra, rb);
+      if (i + 1 < nsteps) step(std::true_type{}, i + 1, xb, db, xa, da, rb, ra);
     }
-    if (i < nsteps) later(i, xb, db, xa, da, rb, ra);
+#pragma unroll 1
+    for (; i + 1 < nsteps; i += 2) {
+      later(i, xa, da, xb, db, ra, rb);
+      later(i + 1, xb, db, xa, da, rb, ra);
+    }
+    if (i < nsteps) later(i, xa, da, xb, db, ra, rb);
     lds_barrier();                        // the product waves' last step
   } else {
     __builtin_amdgcn_s_setprio(3);
     const int ptid = tid - NPT;
-    const int mat = (w >> 1) & 1, kb32 = w & 1;   // (dv | dk) x 32-key block; all D columns
-    f32x16 acc[DB];
+    const int mat = (w >> 1) & 1, half = w & 1;   // (dv | dk) x 64 keys (two 32-key blocks); all D columns
+    f32x16 acc[2][DB];
 #pragma unroll
-    for (int j = 0; j < DB; ++j)
+    for (int kb2 = 0; kb2 < 2; ++kb2)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[j][i] = 0.0f;
+      for (int j = 0; j < DB; ++j)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[kb2][j][i] = 0.0f;
     // Transpose-read offsets (elements).  Rows are queries 16*ks + 8*h + 4*u + i/4; the swizzle
     // depends on the row modulo 16 only, so one offset serves every ks.
-    int xoff[2], yoff[2][DB];
+    int xoff[2][2], yoff[2][DB];
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       const int r = 8 * h + 4 * u + (i16 >> 2);
-      const int xc = 32 * kb32 + 16 * blk + 4 * (i16 & 3);          // key column (elements)
-      xoff[u] = swz_off<BN>(r, xc >> 3) + (xc & 7);
+#pragma unroll
+      for (int kb2 = 0; kb2 < 2; ++kb2) {
+        const int xc = 64 * half + 32 * kb2 + 16 * blk + 4 * (i16 & 3);   // key column (elements)
+        xoff[u][kb2] = swz_off<BKV>(r, xc >> 3) + (xc & 7);
+      }
 #pragma unroll
       for (int j = 0; j < DB; ++j) {
         const int yc = 32 * j + 16 * blk + 4 * (i16 & 3);           // d column (elements)
@@ -525,51 +547,62 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       }
     }
     // Tile staging by the 256 product threads: asynchronous global -> LDS copies straight into
-    // the ring slot, one step ahead of the score waves that will read it.
-    TileCopy<D, BQ, NPT, false> qcopy, gcopy;
+    // the ring slot, well ahead of the score waves that will read it.
+    using Copy = TileCopy<D, BQ, NPT, false>;
+    constexpr int LOADS_PER_TILE = 2 * Copy::NCH;
+    Copy qcopy, gcopy;
     qcopy.init(ptid, qrows.row_bytes);
     gcopy.init(ptid, grows.row_bytes);
     auto fetch = [&](int step) {
-      qcopy.issue(qrows, q_first + step * BQ, Qs + (step & 3) * QTILE);
-      gcopy.issue(grows, q_first + step * BQ, Gs + (step & 3) * QTILE);
+      qcopy.issue(qrows, q_first + step * BQ, Qs + (step & (RING - 1)) * QTILE);
+      gcopy.issue(grows, q_first + step * BQ, Gs + (step & (RING - 1)) * QTILE);
     };
-    fetch(0);
-    fetch(1);
+#pragma unroll
+    for (int sft = 0; sft < AHEAD; ++sft)
+      if (sft < nsteps) fetch(sft);
     wait_loads<0>();
     lds_barrier();
     for (int i = 0; i <= nsteps; ++i) {
-      if (i + 2 < nsteps) fetch(i + 2);
+      if (i + AHEAD < nsteps) fetch(i + AHEAD);
       if (i >= 1) {
-        // acc[key, d] += sum over the 64 queries of step i-1 of X[query][key] * Y[query][d]
+        // acc[key, d] += sum over the 32 queries of step i-1 of X[query][key] * Y[query][d]
         const unsigned short* Xt = (mat ? Zs : Ps) + ((i - 1) & 1) * PTILE;
-        const unsigned short* Yt = (mat ? Qs : Gs) + ((i - 1) & 3) * QTILE;
+        const unsigned short* Yt = (mat ? Qs : Gs) + ((i - 1) & (RING - 1)) * QTILE;
+        // operand reads of both contraction steps first, then their products
+        bf16x8 af[2][2], bf[2][DB];
 #pragma unroll
-        for (int kh = 0; kh < BQ / 32; ++kh) {
-          // operand reads of two contraction steps first, then their 2*DB products
-          bf16x8 af[2], bf[2][DB];
+        for (int ks = 0; ks < BQ / 16; ++ks) {
 #pragma unroll
-          for (int k2 = 0; k2 < 2; ++k2) {
-            const int ks = 2 * kh + k2;
-            af[k2] = lds_tr8(Xt + xoff[0] + 16 * ks * BN, Xt + xoff[1] + 16 * ks * BN);
+          for (int kb2 = 0; kb2 < 2; ++kb2)
+            af[ks][kb2] = lds_tr8(Xt + xoff[0][kb2] + 16 * ks * BKV, Xt + xoff[1][kb2] + 16 * ks * BKV);
 #pragma unroll
-            for (int j = 0; j < DB; ++j)
-              bf[k2][j] = lds_tr8(Yt + yoff[0][j] + 16 * ks * D, Yt + yoff[1][j] + 16 * ks * D);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int k2 = 0; k2 < 2; ++k2)
-#pragma unroll
-            for (int j = 0; j < DB; ++j) acc[j] = mfma32(af[k2], bf[k2][j], acc[j]);
+          for (int j = 0; j < DB; ++j)
+            bf[ks][j] = lds_tr8(Yt + yoff[0][j] + 16 * ks * D, Yt + yoff[1][j] + 16 * ks * D);
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < BQ / 16; ++ks)
+#pragma unroll
+          for (int kb2 = 0; kb2 < 2; ++kb2)
+#pragma unroll
+            for (int j = 0; j < DB; ++j) acc[kb2][j] = mfma32(af[ks][kb2], bf[ks][j], acc[kb2][j]);
       }
-      wait_loads<0>();   // tile i+2 has landed before anyone passes the barrier
+      // Tile i+2 (read by the score waves in step i+1) has landed before anyone passes the
+      // barrier: only the tiles requested after it may still be in flight (loads return in order).
+      const int after = min(i + AHEAD, nsteps - 1) - (i + 2);
+      if (after >= 2) wait_loads<2 * LOADS_PER_TILE>();
+      else if (after == 1) wait_loads<LOADS_PER_TILE>();
+      else wait_loads<0>();
       lds_barrier();
     }
     // (the last barrier of the loop has passed: the p/dz staging buffers are free)
     const View& ov = mat ? a.dk : a.dv;
     __bf16* outb = reinterpret_cast<__bf16*>(ov.ptr) + t.batch * ov.sb + head * ov.sh + tok0 * ov.st;
     unsigned short* scratch = (w & 2 ? Zs : Ps) + (w & 1) * 32 * D;
-    store_block32<D>(scratch, acc, mat ? a.inv_temp : 1.0f, outb, ov.st, kt * BN + 32 * kb32, t.doc_len, lane);
+#pragma unroll
+    for (int kb2 = 0; kb2 < 2; ++kb2)
+      store_block32<D>(scratch, acc[kb2], mat ? a.inv_temp : 1.0f, outb, ov.st, kt * BKV + 64 * half + 32 * kb2,
+                       t.doc_len, lane);
   }
 }
 

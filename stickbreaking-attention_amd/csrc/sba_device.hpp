@@ -22,7 +22,8 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 
 constexpr int BM = 128;  // query rows per workgroup tile (4 waves x 32 rows)
-constexpr int BN = 64;   // keys per KV tile staged in LDS
+constexpr int BN = 64;   // keys per KV tile staged in LDS by the dq pass
+constexpr int BKV = 128;  // keys owned by one workgroup of the dk/dv pass
 constexpr int BT = 32;   // keys per carry-table entry (one MFMA sub-block)
 constexpr int NT = 256;  // threads per workgroup
 

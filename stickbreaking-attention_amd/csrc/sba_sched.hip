@@ -83,7 +83,7 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
     if (i < nd) {
       const int len = dlen[order[i]];
       sq += cdiv(len, BM);
-      skv += cdiv(len, BN);
+      skv += cdiv(len, BKV);
     }
   }
   s_scan_q[tid] = sq;
@@ -104,7 +104,7 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
       const int len = dlen[order[i]];
       qoff[i] = bq; kvoff[i] = bkv;
       bq += cdiv(len, BM);
-      bkv += cdiv(len, BN);
+      bkv += cdiv(len, BKV);
     }
   }
   const int total_q = s_scan_q[SCHED_THREADS - 1], total_kv = s_scan_kv[SCHED_THREADS - 1];

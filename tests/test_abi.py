@@ -39,8 +39,8 @@ def test_workspace_sizes():
     lib = nat.load()
     p = problem()
     sched = lib.sba_schedule_bytes(ctypes.byref(p))
-    # two tile lists (16 B per tile) bounded by tokens/128 + docs and tokens/64 + docs
-    assert 16 * (128 + 8 + 256 + 8) <= sched <= 16 * (128 + 256 + 32) + 1024
+    # two tile lists (16 B per tile): query tiles and key tiles, each bounded by tokens/128 + docs
+    assert 16 * (128 + 8 + 128 + 8) <= sched <= 16 * (128 + 128 + 32) + 1024
     assert lib.sba_table_bytes(ctypes.byref(p)) == 32 * 128 * 16384 * 4
     pf = problem(batch=4, heads=16, tokens=2048, n_docs=0, max_doc_len=2048, head_dim=64,
                  flags=nat.FLAG_FIXED_LENGTH, cu_seqlens=None)
