@@ -184,7 +184,11 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
       if (sub_skip<AC>(k0, qw0)) continue;
       const int64_t tix = (int64_t)(2 * kt + sb) * a.rows_total;
       if (qvalid && h == 0) gtab[tix] = carry_c;
+      // LDS latency under load is several hundred cycles, so every group of operand reads is
+      // issued one phase before the MFMAs that consume it: V rows before the weights are
+      // formed, the transposed K columns before dz is formed.
       float p[16], bt[16];
+      bf16x8 vfr[KS];
       {
         f32x16 x;
 #pragma unroll
@@ -194,30 +198,33 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
         for (int ks = 0; ks < KS; ++ks) kfr[ks] = lds_row8(Kt + 32 * sb * D + roff[ks]);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) x = mfma32(kfr[ks], qf[ks], x);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) vfr[ks] = lds_row8(Vt + 32 * sb * D + roff[ks]);
+        __builtin_amdgcn_sched_barrier(0);
         grad_weights<AC, PROD>(x, a.c, k0, qw0, qrow, h, ce[sb], p, bt);
       }
       bf16x8 zf[2];
+      bf16x8 ktr[2][DB];
       {
         f32x16 da;
 #pragma unroll
         for (int i = 0; i < 16; ++i) da[i] = 0.0f;
-        bf16x8 vfr[KS];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) vfr[ks] = lds_row8(Vt + 32 * sb * D + roff[ks]);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) da = mfma32(vfr[ks], dof[ks], da);
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+          const unsigned short* krow = Kt + (32 * sb + 16 * tt) * D;
+#pragma unroll
+          for (int db = 0; db < DB; ++db) ktr[tt][db] = lds_tr8(krow + toff[0][db], krow + toff[1][db]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         grad_dz(p, bt, da, h, carry_c, dr, zf);
       }
       // dq += dz . K  (K as the B operand: transpose reads along keys)
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-        const unsigned short* krow = Kt + (32 * sb + 16 * tt) * D;
-        bf16x8 kfr[DB];
+      for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-        for (int db = 0; db < DB; ++db) kfr[db] = lds_tr8(krow + toff[0][db], krow + toff[1][db]);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) dqacc[db] = mfma32(zf[tt], kfr[db], dqacc[db]);
-      }
+        for (int db = 0; db < DB; ++db) dqacc[db] = mfma32(zf[tt], ktr[tt][db], dqacc[db]);
     }
     buf ^= 1;
     ce[0] = ce_next[0];
