@@ -111,6 +111,7 @@ struct Timer {
 
 int fill_common(const sba_problem* p, const Sizes& sz, const void* schedule, KArgs* a) {
   if (schedule == nullptr) return SBA_E_NULL;
+  if (reinterpret_cast<uintptr_t>(schedule) & 15) return SBA_E_STRIDE;   // kernels read the header as one 16-byte word
   a->sched = reinterpret_cast<const int*>(schedule);
   a->kv_list_off = SCHED_HDR + 4 * sz.n_q_max;
   a->heads = p->heads;

@@ -81,12 +81,15 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   __shared__ __attribute__((aligned(16))) unsigned short Ks[2 * TILE];
   __shared__ __attribute__((aligned(16))) unsigned short Vs[2 * TILE];
 
+  // Header words and this workgroup's tile are fetched together (the grid never exceeds the
+  // allocated list, so the tile read is safe before the count is known): one round trip.
   const int* sched = a.sched;
-  if (sched[SCHED_STATUS] != 0) return;
   const int slot = blockIdx.x / a.heads;
   const int head = blockIdx.x - slot * a.heads;
-  if (slot >= sched[SCHED_NQ]) return;
+  const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, longest document
   const Tile t = reinterpret_cast<const Tile*>(sched + SCHED_HDR)[slot];
+  asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch));   // keep the tile read above the branch
+  if (hdr.x != 0 || slot >= hdr.y) return;
 
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -269,12 +272,15 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   __shared__ __attribute__((aligned(16))) unsigned short Ps[2 * PTILE];
   __shared__ __attribute__((aligned(16))) unsigned short Zs[2 * PTILE];
 
+  // Header words and this workgroup's tile are fetched together (the grid never exceeds the
+  // allocated list, so the tile read is safe before the count is known): one round trip.
   const int* sched = a.sched;
-  if (sched[SCHED_STATUS] != 0) return;
   const int slot = blockIdx.x / a.heads;
   const int head = blockIdx.x - slot * a.heads;
-  if (slot >= sched[SCHED_NKV]) return;
+  const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, longest document
   const Tile t = reinterpret_cast<const Tile*>(sched + a.kv_list_off)[slot];
+  asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch));   // keep the tile read above the branch
+  if (hdr.x != 0 || slot >= hdr.z) return;
   const int kt = t.idx;
 
   const int tid = threadIdx.x;

@@ -22,12 +22,15 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   unsigned short* const Ks = smem;              // three K tiles
   unsigned short* const Vs = smem + 3 * TILE;   // three V tiles
 
+  // Header words and this workgroup's tile are fetched together (the grid never exceeds the
+  // allocated list, so the tile read is safe before the count is known): one round trip.
   const int* sched = a.sched;
-  if (sched[SCHED_STATUS] != 0) return;
   const int slot = blockIdx.x / a.heads;
   const int head = blockIdx.x - slot * a.heads;
-  if (slot >= sched[SCHED_NQ]) return;
+  const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, longest document
   const Tile t = reinterpret_cast<const Tile*>(sched + SCHED_HDR)[slot];
+  asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch));   // keep the tile read above the branch
+  if (hdr.x != 0 || slot >= hdr.y) return;
 
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
