@@ -33,11 +33,11 @@ namespace sba {
 // p and dz leave as bf16 A-operand fragments: slot s of fragment [tt] is key 16*h + 8*tt + s.
 template <bool AC, bool PROD>
 __device__ __forceinline__ void grad_weights(const f32x16& x, float c, int k0, int qw0, int qrow, int h,
-                                             float carry_e, float (&p)[16], float (&bt)[16]) {
+                                             float carry_e, float (&p)[16], float (&bt)[16], float (&ends)[2]) {
   if (sub_full<AC>(k0, qw0)) {
-    stick_weights<AC, PROD, false, true>(x, c, k0, qrow, h, carry_e, p, bt);
+    stick_weights<AC, PROD, false, true>(x, c, k0, qrow, h, carry_e, p, bt, ends);
   } else {
-    stick_weights<AC, PROD, true, true>(x, c, k0, qrow, h, carry_e, p, bt);
+    stick_weights<AC, PROD, true, true>(x, c, k0, qrow, h, carry_e, p, bt, ends);
   }
 }
 
@@ -45,26 +45,54 @@ __device__ __forceinline__ void grad_weights(const f32x16& x, float c, int k0, i
 //   dz = G - beta C = r C - (C - G) = r * C[i] - C[i-1],
 // so neither G nor beta is formed: the running sum is an fma chain and dz one more fma.  A
 // masked key has p = 0 and r = 1, which gives dz = 0 exactly.
-__device__ __forceinline__ void grad_dz(const float (&p)[16], const float (&r)[16], const f32x16& da, int h,
-                                        float& carry_c, float dr, bf16x8 (&zf)[2]) {
-  float dA[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) dA[i] = da[i] - dr;
-  // this lane's total of G (two partial chains), then both half-waves' totals
-  float t0 = 0.0f, t1 = 0.0f;
-#pragma unroll
-  for (int i = 0; i < 16; i += 2) { t0 = fmaf(p[i], dA[i], t0); t1 = fmaf(p[i + 1], dA[i + 1], t1); }
-  float lo, hi;
-  both_halves(t0 + t1, lo, hi);
-  float cprev = h == 1 ? carry_c + lo : carry_c;   // keys of the h=0 lane come first
+//
+// In product space the subtraction of drem disappears as well.  With ex[i] the stick left on
+// entering key i (so that p[i] = ex[i] - ex[i-1] and r[i] * ex[i] = ex[i-1]) define
+// D[i] = C[i] + drem * ex[i].  Then
+//   D[i] - D[i-1] = p[i] (do.v - drem) + drem p[i] = p[i] do.v          (one fma, no subtraction)
+//   r[i] D[i] - D[i-1] = r[i] C[i] - C[i-1] + drem (r[i] ex[i] - ex[i-1]) = dz[i],
+// so the chain runs on do.v directly and starts from C + drem * (stick after the lane's oldest
+// key); the lane's total of G is sum(p do.v) - drem * sum(p) with sum(p) = ends[0] - ends[1].
+template <bool PROD>
+__device__ __forceinline__ void grad_dz(const float (&p)[16], const float (&r)[16], const f32x16& da,
+                                        const float (&ends)[2], int h, float& carry_c, float dr,
+                                        bf16x8 (&zf)[2]) {
   float dz[16];
+  if constexpr (PROD) {
+    float t0 = 0.0f, t1 = 0.0f;
 #pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const float c = fmaf(p[i], dA[i], cprev);
-    dz[i] = fmaf(r[i], c, -cprev);
-    cprev = c;
+    for (int i = 0; i < 16; i += 2) { t0 = fmaf(p[i], da[i], t0); t1 = fmaf(p[i + 1], da[i + 1], t1); }
+    const float total = fmaf(-dr, ends[0] - ends[1], t0 + t1);   // this lane's sum of G
+    float lo, hi;
+    both_halves(total, lo, hi);
+    const float cstart = h == 1 ? carry_c + lo : carry_c;        // keys of the h=0 lane come first
+    float dprev = fmaf(dr, ends[1], cstart);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float d = fmaf(p[i], da[i], dprev);
+      dz[i] = fmaf(r[i], d, -dprev);
+      dprev = d;
+    }
+    carry_c += lo + hi;
+  } else {
+    float dA[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dA[i] = da[i] - dr;
+    // this lane's total of G (two partial chains), then both half-waves' totals
+    float t0 = 0.0f, t1 = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i += 2) { t0 = fmaf(p[i], dA[i], t0); t1 = fmaf(p[i + 1], dA[i + 1], t1); }
+    float lo, hi;
+    both_halves(t0 + t1, lo, hi);
+    float cprev = h == 1 ? carry_c + lo : carry_c;   // keys of the h=0 lane come first
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float c = fmaf(p[i], dA[i], cprev);
+      dz[i] = fmaf(r[i], c, -cprev);
+      cprev = c;
+    }
+    carry_c += lo + hi;
   }
-  carry_c += lo + hi;
   zf[0] = pack8(dz);
   zf[1] = pack8(dz + 8);
 }
@@ -190,7 +218,7 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
       // LDS latency under load is several hundred cycles, so every group of operand reads is
       // issued one phase before the MFMAs that consume it: V rows before the weights are
       // formed, the transposed K columns before dz is formed.
-      float p[16], bt[16];
+      float p[16], bt[16], ends[2] = {0.0f, 0.0f};
       bf16x8 vfr[KS];
       {
         f32x16 x;
@@ -204,7 +232,7 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) vfr[ks] = lds_row8(Vt + 32 * sb * D + roff[ks]);
         __builtin_amdgcn_sched_barrier(0);
-        grad_weights<AC, PROD>(x, a.c, k0, qw0, qrow, h, ce[sb], p, bt);
+        grad_weights<AC, PROD>(x, a.c, k0, qw0, qrow, h, ce[sb], p, bt, ends);
       }
       bf16x8 zf[2];
       bf16x8 ktr[2][DB];
@@ -221,7 +249,7 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
           for (int db = 0; db < DB; ++db) ktr[tt][db] = lds_tr8(krow + toff[0][db], krow + toff[1][db]);
         }
         __builtin_amdgcn_sched_barrier(0);
-        grad_dz(p, bt, da, h, carry_c, dr, zf);
+        grad_dz<PROD>(p, bt, da, ends, h, carry_c, dr, zf);
       }
       // dq += dz . K  (K as the B operand: transpose reads along keys)
 #pragma unroll
@@ -407,12 +435,12 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       if (DIAG && sub_skip<AC>(k0, qw0)) {
         pf[0] = zero8(); pf[1] = zero8(); zf[0] = zero8(); zf[1] = zero8();
       } else {
-        float p[16], bt[16];
-        if (DIAG) grad_weights<AC, PROD>(xc, a.c, k0, qw0, qrow, h, carry_e, p, bt);
-        else stick_weights<AC, PROD, false, true>(xc, a.c, k0, qrow, h, carry_e, p, bt);
+        float p[16], bt[16], ends[2] = {0.0f, 0.0f};
+        if (DIAG) grad_weights<AC, PROD>(xc, a.c, k0, qw0, qrow, h, carry_e, p, bt, ends);
+        else stick_weights<AC, PROD, false, true>(xc, a.c, k0, qrow, h, carry_e, p, bt, ends);
         pf[0] = pack8(p);
         pf[1] = pack8(p + 8);
-        grad_dz(p, bt, dc, h, carry_c, dr, zf);
+        grad_dz<PROD>(p, bt, dc, ends, h, carry_c, dr, zf);
       }
       stage(i, pf, zf);
       lds_barrier();
@@ -470,34 +498,32 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       post(2);
       // chunk 3: weights and their bf16 fragments
       pre(5);
-      p[0] = ex[0] - ex[0] * r[0];
+      const float after = ex[0] * r[0];       // stick left after this lane's oldest key
+      p[0] = ex[0] - after;
 #pragma unroll
       for (int j = 1; j < 16; ++j) p[j] = ex[j] - ex[j - 1];
       bf16x8 pf[2], zf[2];
       pf[0] = pack8(p);
       pf[1] = pack8(p + 8);
       post(3);
-      // chunk 4: do.v - drem and this lane's total of G
-      pre(6);
-      float dA[16];
-#pragma unroll
-      for (int j = 0; j < 16; ++j) dA[j] = dc[j] - dr;
+      // chunk 4: this lane's total of G = sum(p do.v) - drem sum(p), sum(p) = ex[15] - after
+      pre(4 + LEAD);
       float t0 = 0.0f, t1 = 0.0f;
 #pragma unroll
-      for (int j = 0; j < 16; j += 2) { t0 = fmaf(p[j], dA[j], t0); t1 = fmaf(p[j + 1], dA[j + 1], t1); }
+      for (int j = 0; j < 16; j += 2) { t0 = fmaf(p[j], dc[j], t0); t1 = fmaf(p[j + 1], dc[j + 1], t1); }
       float lo, hi;
-      both_halves(t0 + t1, lo, hi);
-      float cprev = h == 1 ? carry_c + lo : carry_c;
+      both_halves(fmaf(-dr, ex[15] - after, t0 + t1), lo, hi);
+      // chunks 5, 6: D = C + drem * stick runs on do.v directly (see grad_dz); dz = r D[i] - D[i-1]
+      float dprev = fmaf(dr, after, h == 1 ? carry_c + lo : carry_c);
       post(4);
-      // chunks 5, 6: running sum of G and dz = r C[i] - C[i-1]
       float dz[16];
-      pre(7);
+      pre(5 + LEAD);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) { const float cj = fmaf(p[j], dA[j], cprev); dz[j] = fmaf(r[j], cj, -cprev); cprev = cj; }
+      for (int j = 0; j < 8; ++j) { const float dj = fmaf(p[j], dc[j], dprev); dz[j] = fmaf(r[j], dj, -dprev); dprev = dj; }
       post(5);
-      pre(8);
+      pre(6 + LEAD);
 #pragma unroll
-      for (int j = 8; j < 16; ++j) { const float cj = fmaf(p[j], dA[j], cprev); dz[j] = fmaf(r[j], cj, -cprev); cprev = cj; }
+      for (int j = 8; j < 16; ++j) { const float dj = fmaf(p[j], dc[j], dprev); dz[j] = fmaf(r[j], dj, -dprev); dprev = dj; }
       post(6);
       // chunk 7: dz fragments and staging
       pre(9);

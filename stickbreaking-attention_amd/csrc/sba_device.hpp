@@ -171,6 +171,8 @@ __device__ __forceinline__ float prefix_sum32(float (&v)[16], int h, float base)
 //          LOG space: log2 of it (<= 0);  PRODUCT space: the value itself.  Updated in place.
 //   p      out: weights A[q, key(i)]
 //   beta   out (NEED_BETA): 1 - sigmoid(z) (the fraction of the stick a key leaves), 1 where masked
+//   ends   out (PRODUCT space, optional): the stick on entering this lane's newest key and
+//          after its oldest key, {ex[15], ex[0] * r[0]}; their difference is the lane's sum of p
 //
 // Restates compute_block of the upstream Triton kernel
 // (stickbreaking_attention/sb_varlen/sb_varlen_fwd.py:26-78): base-2 softplus
@@ -180,7 +182,8 @@ __device__ __forceinline__ float prefix_sum32(float (&v)[16], int h, float base)
 // ---------------------------------------------------------------------------------------------
 template <bool AC, bool PROD, bool BAND, bool NEED_BETA>
 __device__ __forceinline__ void stick_weights(const f32x16& x, float c, int k0, int qrow, int h,
-                                              float& carry, float (&p)[16], float (&beta)[16]) {
+                                              float& carry, float (&p)[16], float (&beta)[16],
+                                              float* ends = nullptr) {
   // visible keys of a band sub-block: key < qrow (<= with attend_current)  <=>  i < lim
   const int lim = qrow - k0 - 16 * h + (AC ? 1 : 0);
   if constexpr (PROD) {
@@ -196,9 +199,11 @@ __device__ __forceinline__ void stick_weights(const f32x16& x, float c, int k0, 
       if (BAND && !(i < lim)) r[i] = 1.0f;
     }
     carry = suffix_prod32_excl(r, ex, h, carry);
-    p[0] = ex[0] - ex[0] * r[0];
+    const float after = ex[0] * r[0];
+    p[0] = ex[0] - after;
 #pragma unroll
     for (int i = 1; i < 16; ++i) p[i] = ex[i] - ex[i - 1];
+    if (ends != nullptr) { ends[0] = ex[15]; ends[1] = after; }
     if (NEED_BETA) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) beta[i] = r[i];
