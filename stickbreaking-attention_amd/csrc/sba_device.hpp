@@ -261,59 +261,6 @@ __device__ __forceinline__ void store_block32(unsigned short* scratch, const f32
   }
 }
 
-// ---------------------------------------------------------------------------------------------
-// The same product-space arithmetic for an UNMASKED sub-block, cut into chunks with a caller
-// hook between them.  The hook is where a kernel issues MFMAs that do not depend on this
-// sub-block (the chains of the next one, the products of the previous one) and pins their
-// position with a scheduling barrier, so that the matrix core works underneath the VALU
-// stream instead of before or after it.
-//   weights_chunked:  hooks 0..3 after {r[0..7]}, {r[8..15]}, {stick chain}, {p}
-//   dz_chunked:       hooks 0..3 after {do.v - drem, totals}, {dz[0..7]}, {dz[8..15]}, {bf16 pack}
-// ---------------------------------------------------------------------------------------------
-template <class Hook>
-__device__ __forceinline__ void weights_chunked(const f32x16& x, float c, int h, float& carry,
-                                                float (&p)[16], float (&r)[16], Hook&& hook) {
-  float ex[16];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) r[i] = fast_rcp(1.0f + fast_exp2(c * x[i]));
-  hook(0);
-#pragma unroll
-  for (int i = 8; i < 16; ++i) r[i] = fast_rcp(1.0f + fast_exp2(c * x[i]));
-  hook(1);
-  carry = suffix_prod32_excl(r, ex, h, carry);
-  hook(2);
-  p[0] = ex[0] - ex[0] * r[0];
-#pragma unroll
-  for (int i = 1; i < 16; ++i) p[i] = ex[i] - ex[i - 1];
-  hook(3);
-}
-
-template <class Hook>
-__device__ __forceinline__ void dz_chunked(const float (&p)[16], const float (&r)[16], const f32x16& da, int h,
-                                           float& carry_c, float dr, bf16x8 (&zf)[2], Hook&& hook) {
-  float dA[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) dA[i] = da[i] - dr;
-  float t0 = 0.0f, t1 = 0.0f;
-#pragma unroll
-  for (int i = 0; i < 16; i += 2) { t0 = fmaf(p[i], dA[i], t0); t1 = fmaf(p[i + 1], dA[i + 1], t1); }
-  float lo, hi;
-  both_halves(t0 + t1, lo, hi);
-  float cprev = h == 1 ? carry_c + lo : carry_c;   // keys of the h=0 lane come first
-  hook(0);
-  float dz[16];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) { const float ci = fmaf(p[i], dA[i], cprev); dz[i] = fmaf(r[i], ci, -cprev); cprev = ci; }
-  hook(1);
-#pragma unroll
-  for (int i = 8; i < 16; ++i) { const float ci = fmaf(p[i], dA[i], cprev); dz[i] = fmaf(r[i], ci, -cprev); cprev = ci; }
-  hook(2);
-  carry_c += lo + hi;
-  zf[0] = pack8(dz);
-  zf[1] = pack8(dz + 8);
-  hook(3);
-}
-
 // Is the 32-key sub-block starting at k0 entirely invisible / entirely visible to the 32
 // queries starting at qw0?
 template <bool AC>
