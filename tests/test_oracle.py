@@ -184,3 +184,16 @@ def test_make_inputs_is_seeded_and_ordered():
     assert all(torch.equal(x, y) for x, y in zip(a, b))
     g = torch.Generator().manual_seed(1337)
     assert torch.equal(a[0], torch.randn((2, 5, 4), generator=g).to(torch.bfloat16))
+
+
+def test_package_dense_definition_matches_the_oracle():
+    # stickbreaking_attention.sb_ref mirrors the upstream import path (sb_ref.py:8-25); it must
+    # agree with the oracle's dense form, which the closed forms and brute force above pin.
+    from stickbreaking_attention.sb_ref import stickbreaking as dense
+    torch.manual_seed(3)
+    q, k, v = (torch.randn(2, 3, 40, 16, dtype=torch.float64) for _ in range(3))
+    for ac in (False, True):
+        mask, cw = orc.causal_mask_and_weights(40, ac)
+        o1, r1 = dense(q, k, v, mask, cw)
+        o2, r2 = orc.stickbreaking(q, k, v, mask, cw)
+        assert torch.allclose(o1, o2, atol=1e-10) and torch.allclose(r1, r2, atol=1e-10)
