@@ -5,40 +5,36 @@ and private state with PyTorch, pass raw pointers and strides, launch on the cur
 (upstream ``varlen_fwd`` sb_varlen/sb_varlen_fwd.py:413-451, ``varlen_bwd``
 sb_varlen/sb_varlen_bwd.py:484-539, ``_fwd`` sb_attn/sb_fwd.py:139-174, ``_bwd``
 sb_attn/sb_bwd.py:163-205) -- with the device code behind a C ABI instead of a JIT.
-"""
-from __future__ import annotations
 
+Like upstream, every launcher exists twice: as a plain Python function used in eager mode,
+and registered through ``torch.library.custom_op`` under upstream's operator names
+(``stickbreaking_attention::varlen_fwd``, ``::varlen_bwd``, ``::attn_fwd``, ``::attn_bwd``;
+sb_varlen_fwd.py:454, sb_varlen_bwd.py:542, sb_fwd.py:177, sb_bwd.py:208), which is what runs
+while ``torch.compile`` traces.  The registered operators return nothing and write into
+buffers the caller allocated, so they need no shape function.
+"""
 import ctypes
 import math
 import os
-from dataclasses import dataclass
 from typing import Optional, Tuple
 
 import torch
 
 from . import _native as nat
+from .utils import custom_op
 
 # Carry the stick as a running product (2 transcendentals per score) instead of a running
 # log2 sum (3 per score).  Overridable for A/B measurements.
 PRODUCT_SPACE = os.environ.get("SBA_LOG_SPACE", "0") != "1"
 
-# When True every forward reads back the scheduler's status word (one device sync) and raises
-# on malformed cu_seqlens instead of returning untouched outputs.
+# When True every eager forward reads back the scheduler's status word (one device sync) and
+# raises on malformed cu_seqlens instead of returning zero outputs.
 VALIDATE = os.environ.get("SBA_VALIDATE", "0") == "1"
 
 SUPPORTED_HEAD_DIMS = (64, 128)
 
-
-@dataclass
-class Plan:
-    """Everything the kernels need besides the tensors; built once per forward."""
-    problem: nat.SbaProblem
-    schedule: torch.Tensor       # uint8 workspace holding the tile lists
-    fixed: bool
-    table_bytes: int
-    head_dim: int                # padded head_dim the kernels run at
-    orig_head_dim: int
-    keepalive: tuple             # tensors whose pointers live inside `problem`
+# Tile sizes the library's workspace formulas are built on (query tile, dk/dv key tile, table block).
+_BM, _BKV, _BT, _SCHED_HDR = 128, 128, 32, 16
 
 
 def _padded_dim(d: int) -> int:
@@ -48,117 +44,217 @@ def _padded_dim(d: int) -> int:
     raise ValueError(f"head_dim {d} is not supported (maximum {SUPPORTED_HEAD_DIMS[-1]})")
 
 
-def _prep(t: torch.Tensor, dpad: int) -> torch.Tensor:
-    """bf16, head_dim padded with zeros to `dpad`, rows 16-byte aligned."""
+def workspace_sizes(fixed: bool, batch: int, heads: int, tokens: int, n_docs: int, max_doc_len: int) -> Tuple[int, int]:
+    """(schedule bytes, floats of one carry table): the same numbers as ``sba_schedule_bytes`` and
+    ``sba_table_bytes // 4``, computed without touching the library so that they can be
+    evaluated while a graph is being traced (checked against the library in the tests)."""
+    docs = batch if fixed else n_docs
+    rows = (batch if fixed else 1) * tokens
+    n_q = rows // _BM + docs + 1
+    n_kv = rows // _BKV + docs + 1
+    words = _SCHED_HDR + 4 * (n_q + n_kv) + 5 * docs + 2
+    n_tt = -(-max(1, max_doc_len if not fixed else tokens) // _BT)
+    return (4 * words + 255) & ~255, heads * n_tt * rows
+
+
+def _prep(t: torch.Tensor, dpad: int, incoming_grad: bool = False) -> torch.Tensor:
+    """bf16, head_dim padded with zeros to `dpad`, row strides multiples of 8 elements (traceable).
+    The strides of an incoming gradient are not known while a backward is being traced, so
+    there it is simply made contiguous."""
     if t.dtype != torch.bfloat16:
         t = t.to(torch.bfloat16)
     d = t.shape[-1]
     if d != dpad:
         t = torch.nn.functional.pad(t, (0, dpad - d))
-    ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1])
+    if incoming_grad and torch.compiler.is_compiling():
+        return t.contiguous()
+    ok = t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:-1])
     return t if ok else t.contiguous()
 
 
-def make_plan(q: torch.Tensor, fixed: bool, cu_seqlens: Optional[torch.Tensor], max_seqlens: Optional[int],
-              inv_temp: float, attend_current: bool) -> Plan:
+def _aligned(t: torch.Tensor) -> torch.Tensor:
+    """Inputs whose storage offset breaks 16-byte alignment are copied (launch time only)."""
+    return t if t.data_ptr() % 16 == 0 else t.clone(memory_format=torch.contiguous_format)
+
+
+def _problem(q: torch.Tensor, fixed: bool, cu_seqlens: Optional[torch.Tensor], max_doc_len: int,
+             inv_temp: float, attend_current: bool, product: bool):
+    """The ``sba_problem`` of a launch plus the tensors whose pointers it holds."""
+    flags = (nat.FLAG_ATTEND_CURRENT if attend_current else 0) | (nat.FLAG_PRODUCT_SPACE if product else 0)
+    if fixed:
+        B, H, T, d = q.shape
+        return nat.SbaProblem(nat.SBA_BF16, d, H, B, T, 0, T, flags | nat.FLAG_FIXED_LENGTH,
+                              float(inv_temp), None), ()
+    H, T, d = q.shape
+    if cu_seqlens.dtype == torch.int64:
+        flags |= nat.FLAG_CU_INT64
+    cu = cu_seqlens.contiguous()
+    return nat.SbaProblem(nat.SBA_BF16, d, H, 1, T, cu.numel(), max_doc_len, flags, float(inv_temp),
+                          cu.data_ptr() if cu.numel() else None), (cu,)
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return t.data_ptr() if t is not None and t.numel() else None
+
+
+# ---------------------------------------------------------------------------------------------
+# launchers: everything is allocated by the caller
+# ---------------------------------------------------------------------------------------------
+def _launch_fwd(fixed: bool, q, k, v, cu_seqlens, max_doc_len: int, logit_scale: float, attend_current: bool,
+                product: bool, o, rem, table, sched) -> None:
     nat.require_gpu(q)
     lib = nat.load()
-    d = q.shape[-1]
-    dpad = _padded_dim(d)
-    flags = 0
-    if attend_current:
-        flags |= nat.FLAG_ATTEND_CURRENT
-    if PRODUCT_SPACE:
-        flags |= nat.FLAG_PRODUCT_SPACE
-    keep = ()
-    if fixed:
-        B, H, T, _ = q.shape
-        flags |= nat.FLAG_FIXED_LENGTH
-        prob = nat.SbaProblem(nat.SBA_BF16, dpad, H, B, T, 0, T, flags, float(inv_temp), None)
-    else:
-        H, T, _ = q.shape
-        if cu_seqlens.dim() != 1:
-            raise ValueError("cu_seqlens must be 1-d")
-        if cu_seqlens.dtype == torch.int64:
-            flags |= nat.FLAG_CU_INT64
-        elif cu_seqlens.dtype != torch.int32:
-            raise ValueError("cu_seqlens must be int32 or int64")
-        if cu_seqlens.device != q.device:
-            cu_seqlens = cu_seqlens.to(q.device)
-        cu_seqlens = cu_seqlens.contiguous()
-        keep = (cu_seqlens,)
-        bound = T if max_seqlens is None else max(1, min(int(max_seqlens), T))
-        prob = nat.SbaProblem(nat.SBA_BF16, dpad, H, 1, T, cu_seqlens.numel(), bound, flags,
-                              float(inv_temp), cu_seqlens.data_ptr() if cu_seqlens.numel() else None)
-    nbytes = lib.sba_schedule_bytes(ctypes.byref(prob))
-    if nbytes == 0:
-        raise ValueError("invalid problem description for stick-breaking attention")
-    sched = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
-    with torch.cuda.device(q.device):
-        nat.check(lib.sba_build_schedule(ctypes.byref(prob), sched.data_ptr(), nat.stream_ptr(q.device)),
-                  "sba_build_schedule")
-    return Plan(prob, sched, fixed, lib.sba_table_bytes(ctypes.byref(prob)), dpad, d, keep)
-
-
-def check_status(plan: Plan) -> None:
-    """Read the scheduler's status word back (synchronises) and raise on malformed input."""
-    status = int(plan.schedule[:4].view(torch.int32).item())
-    if status != 0:
-        raise ValueError("sb_attn_varlen: " + nat.STATUS_MESSAGES.get(status, f"scheduler status {status}"))
-
-
-def forward(plan: Plan, q, k, v, need_table: bool) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
-    lib = nat.load()
-    fixed = plan.fixed
-    qp, kp, vp = (_prep(t, plan.head_dim) for t in (q, k, v))
-    padded = plan.head_dim != plan.orig_head_dim or q.dtype != torch.bfloat16
-    # Every row is written by the library: rows of documents by the forward kernel, rows that
-    # belong to no document are cleared (upstream leaves those uninitialised).
-    o = torch.empty_like(qp)
-    rem = torch.empty_like(qp[..., 0])
-    table = None
-    if need_table:
-        table = torch.empty(plan.table_bytes // 4, dtype=torch.float32, device=q.device)
+    q, k, v = _aligned(q), _aligned(k), _aligned(v)
+    prob, _keep = _problem(q, fixed, cu_seqlens, max_doc_len, logit_scale, attend_current, product)
+    need, _ = workspace_sizes(fixed, prob.batch, prob.heads, prob.tokens, prob.n_docs, prob.max_doc_len)
+    if sched.numel() * sched.element_size() < need:
+        raise ValueError("schedule workspace too small")
     fn = lib.sba_attn_fwd if fixed else lib.sba_varlen_fwd
     with torch.cuda.device(q.device):
-        code = fn(ctypes.byref(plan.problem), plan.schedule.data_ptr(),
-                  ctypes.byref(nat.view4(qp, fixed)), ctypes.byref(nat.view4(kp, fixed)),
-                  ctypes.byref(nat.view4(vp, fixed)), ctypes.byref(nat.view4(o, fixed)),
-                  ctypes.byref(nat.view4(rem, fixed, per_row=True)),
-                  table.data_ptr() if table is not None else None, nat.stream_ptr(q.device))
+        stream = nat.stream_ptr(q.device)
+        nat.check(lib.sba_build_schedule(ctypes.byref(prob), sched.data_ptr(), stream), "sba_build_schedule")
+        code = fn(ctypes.byref(prob), sched.data_ptr(),
+                  ctypes.byref(nat.view4(q, fixed)), ctypes.byref(nat.view4(k, fixed)),
+                  ctypes.byref(nat.view4(v, fixed)), ctypes.byref(nat.view4(o, fixed)),
+                  ctypes.byref(nat.view4(rem, fixed, per_row=True)), _ptr(table), stream)
     nat.check(code, "sba_attn_fwd" if fixed else "sba_varlen_fwd")
-    if VALIDATE and not fixed:
-        check_status(plan)
-    if padded:
-        o = o[..., :plan.orig_head_dim].to(q.dtype)
-        rem = rem.to(q.dtype)
-    return o, rem, table
 
 
-def backward(plan: Plan, q, k, v, do, drem, table, dkdv_dtype=None):
+def _launch_bwd(fixed: bool, do, dr, q, k, v, cu_seqlens, max_doc_len: int, logit_scale: float,
+                attend_current: bool, product: bool, table, sched, gtab, dq, dk, dv) -> None:
+    nat.require_gpu(q)
     lib = nat.load()
-    fixed = plan.fixed
-    qp, kp, vp, dop = (_prep(t, plan.head_dim) for t in (q, k, v, do))
-    dremp = None
-    if drem is not None:
-        dremp = drem if drem.dtype == torch.bfloat16 else drem.to(torch.bfloat16)
-    padded = plan.head_dim != plan.orig_head_dim or q.dtype != torch.bfloat16
-    dq, dk, dv = torch.empty_like(qp), torch.empty_like(kp), torch.empty_like(vp)
-    gtab = torch.empty(plan.table_bytes // 4, dtype=torch.float32, device=q.device)
+    q, k, v, do = _aligned(q), _aligned(k), _aligned(v), _aligned(do)
+    prob, _keep = _problem(q, fixed, cu_seqlens, max_doc_len, logit_scale, attend_current, product)
     fn = lib.sba_attn_bwd if fixed else lib.sba_varlen_bwd
+    drv = dr if dr is not None and dr.numel() else None
     with torch.cuda.device(q.device):
-        code = fn(ctypes.byref(plan.problem), plan.schedule.data_ptr(),
-                  ctypes.byref(nat.view4(qp, fixed)), ctypes.byref(nat.view4(kp, fixed)),
-                  ctypes.byref(nat.view4(vp, fixed)), ctypes.byref(nat.view4(dop, fixed)),
-                  ctypes.byref(nat.view4(dremp, fixed, per_row=True)),
+        code = fn(ctypes.byref(prob), sched.data_ptr(),
+                  ctypes.byref(nat.view4(q, fixed)), ctypes.byref(nat.view4(k, fixed)),
+                  ctypes.byref(nat.view4(v, fixed)), ctypes.byref(nat.view4(do, fixed)),
+                  ctypes.byref(nat.view4(drv, fixed, per_row=True)),
                   table.data_ptr(), gtab.data_ptr(),
                   ctypes.byref(nat.view4(dq, fixed)), ctypes.byref(nat.view4(dk, fixed)),
                   ctypes.byref(nat.view4(dv, fixed)), nat.stream_ptr(q.device))
     nat.check(code, "sba_attn_bwd" if fixed else "sba_varlen_bwd")
-    if padded:
-        dq = dq[..., :plan.orig_head_dim].to(q.dtype)
-        dk = dk[..., :plan.orig_head_dim].to(k.dtype if dkdv_dtype is None else dkdv_dtype)
-        dv = dv[..., :plan.orig_head_dim].to(v.dtype if dkdv_dtype is None else dkdv_dtype)
+
+
+# The four operators under upstream's names.  Outputs and workspaces are arguments that are
+# written in place; `table` may be empty when no backward will follow.
+@custom_op("varlen_fwd", mutates_args={"o", "rem", "table", "sched"})
+def _compileable_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor,
+                         max_seqlens: int, logit_scale: float, attend_current: bool, product: bool,
+                         o: torch.Tensor, rem: torch.Tensor, table: torch.Tensor, sched: torch.Tensor) -> None:
+    _launch_fwd(False, q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current, product, o, rem, table, sched)
+
+
+@custom_op("varlen_bwd", mutates_args={"gtab", "dq", "dk", "dv"})
+def _compileable_backward(do: torch.Tensor, dr: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                          cu_seqlens: torch.Tensor, max_seqlens: int, logit_scale: float, attend_current: bool,
+                          product: bool, table: torch.Tensor, sched: torch.Tensor, gtab: torch.Tensor,
+                          dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor) -> None:
+    _launch_bwd(False, do, dr, q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current, product,
+                table, sched, gtab, dq, dk, dv)
+
+
+@custom_op("attn_fwd", mutates_args={"o", "rem", "table", "sched"})
+def _compileable_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_scale: float, attend_current: bool,
+                     product: bool, o: torch.Tensor, rem: torch.Tensor, table: torch.Tensor,
+                     sched: torch.Tensor) -> None:
+    _launch_fwd(True, q, k, v, None, q.shape[2], logit_scale, attend_current, product, o, rem, table, sched)
+
+
+@custom_op("attn_bwd", mutates_args={"gtab", "dq", "dk", "dv"})
+def _compileable_bwd(do: torch.Tensor, dr: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                     logit_scale: float, attend_current: bool, product: bool, table: torch.Tensor,
+                     sched: torch.Tensor, gtab: torch.Tensor, dq: torch.Tensor, dk: torch.Tensor,
+                     dv: torch.Tensor) -> None:
+    _launch_bwd(True, do, dr, q, k, v, None, q.shape[2], logit_scale, attend_current, product,
+                table, sched, gtab, dq, dk, dv)
+
+
+# ---------------------------------------------------------------------------------------------
+# what the autograd functions call
+# ---------------------------------------------------------------------------------------------
+def _check_cu(cu_seqlens: torch.Tensor, like: torch.Tensor) -> torch.Tensor:
+    if cu_seqlens.dim() != 1:
+        raise ValueError("cu_seqlens must be 1-d")
+    if cu_seqlens.dtype not in (torch.int32, torch.int64):
+        raise ValueError("cu_seqlens must be int32 or int64")
+    if cu_seqlens.device != like.device:
+        cu_seqlens = cu_seqlens.to(like.device)
+    return cu_seqlens
+
+
+def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, attend_current: bool,
+            need_table: bool):
+    """Returns (o, rem, state); ``state`` = (table, sched, cu_seqlens, max_doc_len, product) is what
+    the backward needs (upstream keeps its fp32 ``neg_log_acc`` there)."""
+    nat.require_gpu(q)
+    d = q.shape[-1]
+    dpad = _padded_dim(d)
+    product = PRODUCT_SPACE
+    qp, kp, vp = (_prep(t, dpad) for t in (q, k, v))
+    if fixed:
+        B, H, T, _ = qp.shape
+        n_docs, max_len, cu = 0, T, None
+    else:
+        H, T, _ = qp.shape
+        B = 1
+        cu = _check_cu(cu_seqlens, q)
+        n_docs = cu.numel()
+        max_len = T if max_seqlens is None else max(1, min(int(max_seqlens), T))
+    sched_bytes, table_floats = workspace_sizes(fixed, B, H, T, n_docs, max_len)
+    # Every row is written by the library: rows of documents by the forward kernel, rows that
+    # belong to no document are cleared (upstream leaves those uninitialised).
+    o = torch.empty_like(qp)
+    rem = torch.empty_like(qp[..., 0])
+    table = torch.empty(table_floats if need_table else 0, dtype=torch.float32, device=q.device)
+    sched = torch.empty(sched_bytes, dtype=torch.uint8, device=q.device)
+    if fixed:
+        _compileable_fwd(qp, kp, vp, float(inv_temp), bool(attend_current), product, o, rem, table, sched)
+    else:
+        _compileable_forward(qp, kp, vp, cu, max_len, float(inv_temp), bool(attend_current), product,
+                             o, rem, table, sched)
+        if VALIDATE and not torch.compiler.is_compiling():
+            check_status(sched)
+    if dpad != d or q.dtype != torch.bfloat16:
+        o = o[..., :d].to(q.dtype)
+        rem = rem.to(q.dtype)
+    return o, rem, (table, sched, cu, max_len, product)
+
+
+def check_status(sched: torch.Tensor) -> None:
+    """Read the scheduler's status word back (synchronises) and raise on malformed input."""
+    status = int(sched[:4].view(torch.int32).item())
+    if status != 0:
+        raise ValueError("sb_attn_varlen: " + nat.STATUS_MESSAGES.get(status, f"scheduler status {status}"))
+
+
+def run_backward(q, k, v, do, drem, fixed: bool, state, inv_temp: float, attend_current: bool, dkdv_dtype=None):
+    table, sched, cu, max_len, product = state
+    d = q.shape[-1]
+    dpad = _padded_dim(d)
+    qp, kp, vp = (_prep(t, dpad) for t in (q, k, v))
+    dop = _prep(do, dpad, incoming_grad=True)
+    if drem is None:
+        dremp = torch.empty(0, dtype=torch.bfloat16, device=q.device)
+    else:
+        dremp = drem if drem.dtype == torch.bfloat16 else drem.to(torch.bfloat16)
+        if torch.compiler.is_compiling():
+            dremp = dremp.contiguous()
+    dq, dk, dv = torch.empty_like(qp), torch.empty_like(kp), torch.empty_like(vp)
+    gtab = torch.empty_like(table)
+    if fixed:
+        _compileable_bwd(dop, dremp, qp, kp, vp, float(inv_temp), bool(attend_current), product,
+                         table, sched, gtab, dq, dk, dv)
+    else:
+        _compileable_backward(dop, dremp, qp, kp, vp, cu, max_len, float(inv_temp), bool(attend_current),
+                              product, table, sched, gtab, dq, dk, dv)
+    if dpad != d or q.dtype != torch.bfloat16:
+        dq = dq[..., :d].to(q.dtype)
+        dk = dk[..., :d].to(k.dtype if dkdv_dtype is None else dkdv_dtype)
+        dv = dv[..., :d].to(v.dtype if dkdv_dtype is None else dkdv_dtype)
     return dq, dk, dv
 
 

@@ -17,14 +17,11 @@ BWD_BLOCK_N = 64
 
 
 def _fwd(q, k, v, logit_scale, attend_current=False, no_grad=False):
-    plan = _ops.make_plan(q, True, None, None, logit_scale, attend_current)
-    o, rem, table = _ops.forward(plan, q, k, v, need_table=not no_grad)
-    return o, rem, (plan, table)
+    return _ops.run_forward(q, k, v, True, None, None, logit_scale, attend_current, need_table=not no_grad)
 
 
-def _bwd(do, dr, q, k, v, state, logit_scale=None, attend_current=None):
-    plan, table = state
-    return _ops.backward(plan, q, k, v, do, dr, table)
+def _bwd(do, dr, q, k, v, state, logit_scale, attend_current=False):
+    return _ops.run_backward(q, k, v, do, dr, True, state, logit_scale, attend_current)
 
 
 class StickBreakingAttention(torch.autograd.Function):
@@ -33,18 +30,19 @@ class StickBreakingAttention(torch.autograd.Function):
     def forward(ctx, q, k, v, inv_temp, attend_current=False):
         no_grad = not any(ctx.needs_input_grad[:3])
         o, rem, state = _fwd(q, k, v, logit_scale=inv_temp, attend_current=attend_current, no_grad=no_grad)
-        plan, table = state
-        if table is not None:
-            ctx.save_for_backward(q, k, v, table)
-        ctx.plan = plan
+        table, sched, _cu, max_len, product = state
+        ctx.save_for_backward(q, k, v, table, sched)
         ctx.logit_scale = inv_temp
+        ctx.max_seqlens = max_len
         ctx.attend_current = attend_current
+        ctx.product = product
         return o, rem
 
     @staticmethod
     def backward(ctx, do, drem):
-        q, k, v, table = ctx.saved_tensors
-        dq, dk, dv = _bwd(do, drem, q, k, v, (ctx.plan, table))
+        q, k, v, table, sched = ctx.saved_tensors
+        state = (table, sched, None, ctx.max_seqlens, ctx.product)
+        dq, dk, dv = _bwd(do, drem, q, k, v, state, ctx.logit_scale, ctx.attend_current)
         return dq, dk, dv, None, None
 
 

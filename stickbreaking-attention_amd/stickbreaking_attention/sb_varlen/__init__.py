@@ -18,15 +18,13 @@ BWD_BLOCK_N = 64
 
 def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=False, no_grad=False):
     """Host launcher of the forward; returns (o, rem, state) where ``state`` is what the
-    backward needs (plan + carry table) -- upstream returns its fp32 ``neg_log_acc`` there."""
-    plan = _ops.make_plan(q, False, cu_seqlens, max_seqlens, logit_scale, attend_current)
-    o, rem, table = _ops.forward(plan, q, k, v, need_table=not no_grad)
-    return o, rem, (plan, table)
+    backward needs (carry table, schedule, ...) -- upstream returns its fp32 ``neg_log_acc`` there."""
+    return _ops.run_forward(q, k, v, False, cu_seqlens, max_seqlens, logit_scale, attend_current,
+                        need_table=not no_grad)
 
 
-def varlen_bwd(do, dr, q, k, v, state, logit_scale=None, attend_current=None):
-    plan, table = state
-    return _ops.backward(plan, q, k, v, do, dr, table)
+def varlen_bwd(do, dr, q, k, v, state, logit_scale, attend_current=False):
+    return _ops.run_backward(q, k, v, do, dr, False, state, logit_scale, attend_current)
 
 
 class StickBreakingAttention(torch.autograd.Function):
@@ -36,19 +34,19 @@ class StickBreakingAttention(torch.autograd.Function):
         no_grad = not any(ctx.needs_input_grad[:3])
         o, rem, state = varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale=inv_temp,
                                    attend_current=attend_current, no_grad=no_grad)
-        plan, table = state
-        if table is not None:
-            ctx.save_for_backward(q, k, v, table, cu_seqlens)
-        ctx.plan = plan
+        table, sched, cu, max_len, product = state
+        ctx.save_for_backward(q, k, v, table, sched, cu)
         ctx.logit_scale = inv_temp
-        ctx.max_seqlens = max_seqlens
+        ctx.max_seqlens = max_len
         ctx.attend_current = attend_current
+        ctx.product = product
         return o, rem
 
     @staticmethod
     def backward(ctx, do, drem):
-        q, k, v, table, _cu = ctx.saved_tensors
-        dq, dk, dv = varlen_bwd(do, drem, q, k, v, (ctx.plan, table))
+        q, k, v, table, sched, cu = ctx.saved_tensors
+        state = (table, sched, cu, ctx.max_seqlens, ctx.product)
+        dq, dk, dv = varlen_bwd(do, drem, q, k, v, state, ctx.logit_scale, ctx.attend_current)
         return dq, dk, dv, None, None, None, None
 
 

@@ -90,3 +90,34 @@ def test_missing_library_raises(monkeypatch):
     monkeypatch.setattr(nat, "LIB_PATH", "/nonexistent/libsba.so")
     with pytest.raises(RuntimeError, match="libsba.so not found"):
         nat.load()
+
+
+@pytest.mark.parametrize("kw", [
+    dict(),                                                           # C3
+    dict(head_dim=64, tokens=16384, n_docs=207, max_doc_len=256),     # many short documents
+    dict(tokens=65536, n_docs=7, max_doc_len=32768),
+    dict(tokens=300, n_docs=1, max_doc_len=300, heads=2),
+    dict(tokens=130, n_docs=0, max_doc_len=130, heads=3),
+    dict(batch=4, heads=16, tokens=2048, n_docs=0, max_doc_len=2048, head_dim=64, fixed=True),
+    dict(batch=2, heads=7, tokens=500, n_docs=0, max_doc_len=500, head_dim=64, fixed=True),
+])
+def test_python_workspace_formula_matches_the_library(kw):
+    # _ops.workspace_sizes restates sba_schedule_bytes / sba_table_bytes so that buffer sizes can
+    # be computed while torch.compile traces; the two must never drift apart.
+    from stickbreaking_attention import _ops
+    lib = nat.load()
+    kw = dict(kw)
+    fixed = kw.pop("fixed", False)
+    if fixed:
+        kw.update(flags=nat.FLAG_FIXED_LENGTH, cu_seqlens=None)
+    p = problem(**kw)
+    sched, table = _ops.workspace_sizes(fixed, p.batch, p.heads, p.tokens, p.n_docs, p.max_doc_len)
+    assert sched == lib.sba_schedule_bytes(ctypes.byref(p))
+    assert 4 * table == lib.sba_table_bytes(ctypes.byref(p))
+
+
+def test_operators_are_registered_under_the_upstream_names():
+    import torch
+    import stickbreaking_attention  # noqa: F401
+    for name in ("varlen_fwd", "varlen_bwd", "attn_fwd", "attn_bwd"):
+        assert hasattr(torch.ops.stickbreaking_attention, name)
