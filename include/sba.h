@@ -98,7 +98,7 @@ size_t sba_table_bytes(const sba_problem* p);
 
 /* ---- schedule --------------------------------------------------------------------------- */
 
-/* Builds, on the device, the list of 128-row query tiles and 64-key KV tiles from
+/* Builds, on the device, the list of 128-row query tiles and 128-key KV tiles from
  * cu_seqlens (documents sorted longest first, tiles of a document newest first) and validates
  * cu_seqlens.  `schedule` must hold sba_schedule_bytes() bytes and be 16-byte aligned.  The first int32 of the
  * workspace is a status word (0 = ok, else SBA_STATUS_*), readable by the caller after the

@@ -16,7 +16,7 @@ struct KArgs {
   float* gtab;                 // gradient prefix table (backward scratch)
   int heads;
   int tokens;                  // tokens per batch entry
-  int n_tt;                    // table tiles per row = ceil(max_doc_len / BN)
+  int n_tt;                    // table blocks per row = ceil(max_doc_len / 32)
   int64_t rows_total;          // batch * tokens
   float c;                     // inv_temp * log2(e)
   float inv_temp;

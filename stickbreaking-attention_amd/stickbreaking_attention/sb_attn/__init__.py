@@ -10,8 +10,9 @@ import torch
 
 from .. import _ops
 
+# Tile sizes of the HIP kernels (upstream exposes its Triton block sizes under these names).
 FWD_BLOCK_M = 128
-FWD_BLOCK_N = 64
+FWD_BLOCK_N = 32
 BWD_BLOCK_M = 128
 BWD_BLOCK_N = 64
 
