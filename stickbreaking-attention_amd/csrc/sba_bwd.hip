@@ -394,10 +394,10 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
         da = mfma32(vf[ks], gfr[ks], da);
       }
     };
-    auto stage = [&](int step, const bf16x8 (&pf)[2], const bf16x8 (&zf)[2]) {
+    auto stage = [&](int parity, const bf16x8 (&pf)[2], const bf16x8 (&zf)[2]) {
       // p and dz as [query][key]: fragment tt is 8 consecutive keys = one 16-byte chunk
-      unsigned short* Pt = Ps + (step & 1) * PTILE;
-      unsigned short* Zt = Zs + (step & 1) * PTILE;
+      unsigned short* Pt = Ps + parity * PTILE;
+      unsigned short* Zt = Zs + parity * PTILE;
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt) {
         const int chunk = 4 * sb + 2 * h + tt;
@@ -442,7 +442,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
         pf[1] = pack8(p + 8);
         grad_dz<PROD>(p, bt, dc, ends, h, carry_c, dr, zf);
       }
-      stage(i, pf, zf);
+      stage(i & 1, pf, zf);
       lds_barrier();
       __builtin_amdgcn_sched_barrier(0);   // keep the consumers of the requested values down here
       carry_e = ncarry_e; carry_c = ncarry_c; dr = ndr;
@@ -452,11 +452,17 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     // VALU work on block i is cut into 8 chunks and the 2*KS chain MFMAs of block i+1 are
     // issued between them (operand reads two chunks ahead), each position pinned with a
     // scheduling barrier so that the matrix core runs underneath the VALU stream.
-    auto bulk = [&](int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& req, const Raw& due) {
+    // SLOT >= 0: the ring slot of tile i+1 (and with it the p/dz buffer, SLOT and i have opposite
+    // parity) is a compile-time constant, so every LDS address is a fixed register plus an
+    // immediate; SLOT < 0: taken from i at run time.
+    auto bulk = [&](auto slot_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& req, const Raw& due) {
+      constexpr int SLOT = decltype(slot_tag)::value;
       constexpr int NCHUNK = 8, PER = 2 * KS / NCHUNK;
       request(i + 3, req);
-      const unsigned short* Qt = Qs + ((i + 1) & (RING - 1)) * QTILE;
-      const unsigned short* Gt = Gs + ((i + 1) & (RING - 1)) * QTILE;
+      const int slot8 = SLOT >= 0 ? SLOT : ((i + 1) & (RING - 1));
+      const int parity = SLOT >= 0 ? ((SLOT + 1) & 1) : (i & 1);
+      const unsigned short* Qt = Qs + slot8 * QTILE;
+      const unsigned short* Gt = Gs + slot8 * QTILE;
 #pragma unroll
       for (int j = 0; j < 16; ++j) { xn[j] = 0.0f; dn[j] = 0.0f; }
       // Operand reads run LEAD chunks ahead of the MFMAs that consume them (LDS latency under
@@ -529,7 +535,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       pre(9);
       zf[0] = pack8(dz);
       zf[1] = pack8(dz + 8);
-      stage(i, pf, zf);
+      stage(parity, pf, zf);
       post(7);
       lds_barrier();
       __builtin_amdgcn_sched_barrier(0);
@@ -537,8 +543,8 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       carry_e = ncarry_e; dr = ndr;
       settle(i + 2, due, ncarry_e, ncarry_c, ndr);
     };
-    auto later = [&](int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& req, const Raw& due) {
-      if constexpr (PROD) bulk(i, xc, dc, xn, dn, req, due);
+    auto later = [&](auto slot_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& req, const Raw& due) {
+      if constexpr (PROD) bulk(slot_tag, i, xc, dc, xn, dn, req, due);
       else step(std::false_type{}, i, xc, dc, xn, dn, req, due);
     };
     f32x16 xa, da, xb, db;
@@ -550,12 +556,28 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       step(std::true_type{}, i, xa, da, xb, db, ra, rb);
       if (i + 1 < nsteps) step(std::true_type{}, i + 1, xb, db, xa, da, rb, ra);
     }
+    // Whole turns of the ring with static slots (i is a multiple of BKV/BQ = 4 here, so tile
+    // i+1 sits in slot 5, 6, 7, 0, ...), then the remaining steps with run-time slots.
+    using std::integral_constant;
+    if (i == BKV / BQ) {
+#pragma unroll 1
+      for (; i + RING <= nsteps; i += RING) {
+        later(integral_constant<int, 5>{}, i, xa, da, xb, db, ra, rb);
+        later(integral_constant<int, 6>{}, i + 1, xb, db, xa, da, rb, ra);
+        later(integral_constant<int, 7>{}, i + 2, xa, da, xb, db, ra, rb);
+        later(integral_constant<int, 0>{}, i + 3, xb, db, xa, da, rb, ra);
+        later(integral_constant<int, 1>{}, i + 4, xa, da, xb, db, ra, rb);
+        later(integral_constant<int, 2>{}, i + 5, xb, db, xa, da, rb, ra);
+        later(integral_constant<int, 3>{}, i + 6, xa, da, xb, db, ra, rb);
+        later(integral_constant<int, 4>{}, i + 7, xb, db, xa, da, rb, ra);
+      }
+    }
 #pragma unroll 1
     for (; i + 1 < nsteps; i += 2) {
-      later(i, xa, da, xb, db, ra, rb);
-      later(i + 1, xb, db, xa, da, rb, ra);
+      later(integral_constant<int, -1>{}, i, xa, da, xb, db, ra, rb);
+      later(integral_constant<int, -1>{}, i + 1, xb, db, xa, da, rb, ra);
     }
-    if (i < nsteps) later(i, xa, da, xb, db, ra, rb);
+    if (i < nsteps) later(integral_constant<int, -1>{}, i, xa, da, xb, db, ra, rb);
     lds_barrier();                        // the product waves' last step
   } else {
     __builtin_amdgcn_s_setprio(3);
