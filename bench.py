@@ -28,6 +28,8 @@ MEASURED_TRAFFIC_BYTES = {"c3": {"fwd_kernel": 1.151e9, "bwd_dq_kernel": 1.089e9
 
 
 def workload(name):
+    if name == "c2":   # fixed-length sb_attn: batch 4 x 16 heads x 2048 tokens x d=64, every (batch, head) one document
+        return [2048] * 4, dict(H=16, d=64, scale=1.0, zero_start=False, backward=True, fixed=True)
     with open(os.path.join(ROOT, "tests", "golden", "doc_lengths.json")) as f:
         lengths = json.load(f)[name]
     cfg = {"c3": dict(H=32, d=128, scale=1.0, zero_start=False, backward=True),
@@ -66,7 +68,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c3", choices=["c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
     ap.add_argument("--lengths", default=None,
                     help="comma-separated document lengths replacing the workload's own (shape sweeps; "
                          "heads, head_dim and scaling stay those of --workload)")
@@ -81,7 +83,7 @@ def main():
 
     import torch
     from oracle import sb_oracle as orc
-    from stickbreaking_attention import _native, _ops, sb_attn_varlen
+    from stickbreaking_attention import _native, _ops, sb_attn, sb_attn_varlen
     if args.log_space:
         _ops.PRODUCT_SPACE = False
     lib = _native.load()
@@ -92,7 +94,12 @@ def main():
         lengths = [int(x) for x in args.lengths.split(",")]
         args.workload = f"{args.workload}/custom"
     H, d, T = cfg["H"], cfg["d"], sum(lengths)
-    q, k, v, do = (t.to(dev) for t in orc.make_inputs((H, T, d), 1337, scale=cfg["scale"]))
+    fixed = cfg.get("fixed", False)
+    if fixed:
+        B, T = len(lengths), lengths[0]
+        q, k, v, do = (t.to(dev) for t in orc.make_inputs((B, H, T, d), 1337, scale=cfg["scale"]))
+    else:
+        q, k, v, do = (t.to(dev) for t in orc.make_inputs((H, T, d), 1337, scale=cfg["scale"]))
     cu = torch.tensor(lengths, dtype=torch.int64).cumsum(0)
     if cfg["zero_start"]:
         cu = torch.cat([torch.zeros(1, dtype=torch.int64), cu])
@@ -102,16 +109,21 @@ def main():
     if backward:
         q.requires_grad_(); k.requires_grad_(); v.requires_grad_()
 
+    def attention():
+        if fixed:
+            return sb_attn(q, k, v)
+        return sb_attn_varlen(q, k, v, cu, max_len, zero_start=cfg["zero_start"])
+
     def step():
         if backward:
-            o, rem = sb_attn_varlen(q, k, v, cu, max_len, zero_start=cfg["zero_start"])
+            o, rem = attention()
             return torch.autograd.grad(o, (q, k, v), do)
         with torch.no_grad():
-            return sb_attn_varlen(q, k, v, cu, max_len, zero_start=cfg["zero_start"])
+            return attention()
 
     def fwd_only():
         with torch.no_grad():
-            return sb_attn_varlen(q, k, v, cu, max_len, zero_start=cfg["zero_start"])
+            return attention()
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
@@ -170,8 +182,9 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: sb_attn_varlen {'fwd+bwd' if backward else 'fwd'} H={H} d={d} "
-                               f"T={T} in {len(lengths)} documents (tests/golden/doc_lengths.json), N(0,1)*{cfg['scale']}",
+        "config": {"workload": (f"{args.workload}: sb_attn fwd+bwd B={len(lengths)} H={H} T={T} d={d}, N(0,1)" if fixed else
+                               f"{args.workload}: sb_attn_varlen {'fwd+bwd' if backward else 'fwd'} H={H} d={d} "
+                               f"T={T} in {len(lengths)} documents (tests/golden/doc_lengths.json), N(0,1)*{cfg['scale']}"),
                    "carry": "product" if _ops.PRODUCT_SPACE else "log2-sum", "sum_L2": sum(l * l for l in lengths)},
         "fwd_ms": ms_fwd, "fwd_tflops": 4.0 * d * pairs / (ms_fwd * 1e-3) / 1e12,
         "frac_of_bf16_peak": total_flops / (ms_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
