@@ -196,8 +196,10 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   float ce[2], ce_next[2];
   carries(0, ce);
 
-  int buf = 0;
-  for (int kt = 0; kt <= kt_last; ++kt) {
+  // One tile step; the buffer index is a compile-time constant so that every LDS address is a
+  // fixed register plus an immediate.
+  auto tile = [&](auto buf_tag, const int kt) {
+    constexpr int buf = decltype(buf_tag)::value;
     // tile kt has landed and every wave is done with the tile before it
     wait_loads<0>();
     lds_barrier();
@@ -257,9 +259,14 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
 #pragma unroll
         for (int db = 0; db < DB; ++db) dqacc[db] = mfma32(zf[tt], ktr[tt][db], dqacc[db]);
     }
-    buf ^= 1;
     ce[0] = ce_next[0];
     ce[1] = ce_next[1];
+  };
+  for (int kt = 0;;) {
+    tile(std::integral_constant<int, 0>{}, kt);
+    if (++kt > kt_last) break;
+    tile(std::integral_constant<int, 1>{}, kt);
+    if (++kt > kt_last) break;
   }
 
   lds_barrier();   // every wave is done with the K/V tiles: their memory becomes the dq staging area
