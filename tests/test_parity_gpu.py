@@ -79,6 +79,17 @@ def test_config1_shape(product_space, monkeypatch):
     check_all(run_varlen(q, k, v, do, [512]), oracle_varlen(q, k, v, do, [512]))
 
 
+@pytest.mark.parametrize("ac", [False, True])
+def test_log_space_carry_on_long_documents(ac, monkeypatch):
+    """The log2-sum variant of the kernels (the reference's formulation) over documents long enough
+    to wrap the dk/dv pass's tile ring several times, head_dim 128."""
+    from stickbreaking_attention import _ops
+    monkeypatch.setattr(_ops, "PRODUCT_SPACE", False)
+    lengths = [1100, 437]
+    q, k, v, do = orc.make_inputs((2, sum(lengths), 128), 77)
+    check_all(run_varlen(q, k, v, do, lengths, ac), oracle_varlen(q, k, v, do, lengths, ac))
+
+
 @pytest.mark.parametrize("lengths", [[1], [2], [3, 1, 1, 2], [63, 64, 65, 127, 128, 129, 1, 31, 33], [257, 640]])
 @pytest.mark.parametrize("ac", [False, True])
 @pytest.mark.parametrize("d", [64, 128])
