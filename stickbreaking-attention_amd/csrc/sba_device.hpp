@@ -230,6 +230,61 @@ __device__ __forceinline__ void stick_weights(const f32x16& x, float c, int k0, 
 }
 
 // ---------------------------------------------------------------------------------------------
+// Forward-only form of the product-space weights with a quarter of the reciprocals.
+//
+// With e = 2^z (the odds of taking the stick) and t = 1 + e, a key divides the stick by t and
+// takes the difference.  For a group of four keys only ONE reciprocal is needed: the stick
+// after the group's oldest key is (stick before the group) / (t0 t1 t2 t3), and the stick after
+// key i of the group is that times the t of the group's older keys (a running product).  A transcendental costs about four ordinary instructions on this machine, so
+// 16 exp2 + 4 rcp per lane beat 16 exp2 + 16 rcp although a few more multiplies are needed.
+// The backward kernels need r = 1/t for every key and keep the plain form (stick_weights).
+//
+// The odds are clamped at 2^30 so that a product of four t stays finite (beta = 1 - 2^-30 there,
+// which in fp32 is 1); a masked key has e = 0: t = 1, p = 0.
+// ---------------------------------------------------------------------------------------------
+template <bool AC, bool BAND>
+__device__ __forceinline__ void stick_weights_fwd(const f32x16& x, float c, int k0, int qrow, int h,
+                                                  float& carry, float (&p)[16]) {
+  const int lim = qrow - k0 - 16 * h + (AC ? 1 : 0);   // visible keys of a band block: i < lim
+  // per group of four keys (register i = key 16*h + i, so a smaller i is an older key):
+  // u1, u2, u3 = running products of t from the oldest key, inv = 1 / (product of all four)
+  float u1[4], u2[4], u3[4], inv[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    float t[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int i = 4 * g + j;
+      const float e = fast_exp2(fminf(c * x[i], 30.0f));
+      t[j] = (BAND && !(i < lim)) ? 1.0f : 1.0f + e;
+    }
+    u1[g] = t[0];
+    u2[g] = u1[g] * t[1];
+    u3[g] = u2[g] * t[2];
+    inv[g] = fast_rcp(u3[g] * t[3]);
+  }
+  const float total = (inv[0] * inv[1]) * (inv[2] * inv[3]);   // what this lane's 16 keys leave of a stick
+  float lo, hi;
+  both_halves(total, lo, hi);
+  // keys of the h=1 lane (16..31) are newer than those of the h=0 lane
+  float s = h == 0 ? carry * hi : carry;
+  // Newest group first.  With s the stick after the group's oldest key, the stick after key j
+  // of the group is s * u_j and the stick before its newest key is the previous s; a key's
+  // weight is the difference of the stick before and after it.
+#pragma unroll
+  for (int g = 3; g >= 0; --g) {
+    const float before = s;
+    s *= inv[g];
+    const float a1 = s * u1[g], a2 = s * u2[g], a3 = s * u3[g];
+    p[4 * g] = a1 - s;
+    p[4 * g + 1] = a2 - a1;
+    p[4 * g + 2] = a3 - a2;
+    p[4 * g + 3] = before - a3;
+  }
+  carry *= lo * hi;
+}
+
+// ---------------------------------------------------------------------------------------------
 // Epilogue: one wave writes its 32 x D block of fp32 accumulators (lane = column n of a 32-wide
 // block, register i = row 8*(i/4) + 4*h + i%4) to global memory as bf16.  Storing straight from
 // that layout would take 16*D/32 two-byte stores per lane; instead the block goes through a

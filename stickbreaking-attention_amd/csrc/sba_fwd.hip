@@ -124,11 +124,14 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) x = mfma32(kfr[ks], qf[ks], x);
     }
-    float p[16], unused[16];
-    if (sub_full<AC>(k0, qw0)) {
-      stick_weights<AC, PROD, false, false>(x, a.c, k0, qrow, h, carry, p, unused);
+    float p[16];
+    if constexpr (PROD) {
+      if (sub_full<AC>(k0, qw0)) stick_weights_fwd<AC, false>(x, a.c, k0, qrow, h, carry, p);
+      else stick_weights_fwd<AC, true>(x, a.c, k0, qrow, h, carry, p);
     } else {
-      stick_weights<AC, PROD, true, false>(x, a.c, k0, qrow, h, carry, p, unused);
+      float unused[16];
+      if (sub_full<AC>(k0, qw0)) stick_weights<AC, PROD, false, false>(x, a.c, k0, qrow, h, carry, p, unused);
+      else stick_weights<AC, PROD, true, false>(x, a.c, k0, qrow, h, carry, p, unused);
     }
     // P as the A operand of O = P.V: slot s of step tt is key 16*h + 8*tt + s, which the
     // permuted tile keeps in LDS row 16*tt + 8*(s/4) + 4*h + s%4.
