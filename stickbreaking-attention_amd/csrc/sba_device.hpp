@@ -149,18 +149,6 @@ __device__ __forceinline__ float suffix_sum32(float (&v)[16], int h, float base)
   return lo + hi;
 }
 
-// v[i] <- base + sum of v over keys <= key(i).  Returns the plain total over the 32 keys.
-__device__ __forceinline__ float prefix_sum32(float (&v)[16], int h, float base) {
-  const float t = (((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]))) +
-                  (((v[8] + v[9]) + (v[10] + v[11])) + ((v[12] + v[13]) + (v[14] + v[15])));
-  float lo, hi;
-  both_halves(t, lo, hi);
-  v[0] += h == 1 ? base + lo : base;
-#pragma unroll
-  for (int i = 1; i < 16; ++i) v[i] += v[i - 1];
-  return lo + hi;
-}
-
 // ---------------------------------------------------------------------------------------------
 // Stick-breaking weights of one 32-key sub-block for the lane's query.
 //
@@ -357,32 +345,6 @@ __device__ __forceinline__ bf16x8 load_frag(const Rows& r, int row, int col_byte
   return __builtin_bit_cast(bf16x8, load16(r, row, col_bytes));
 }
 
-// Cooperative load of ROWS x D bf16 (16 bytes per thread per step) by THREADS threads.
-// KEYS = true: the tile holds keys and register slot (m, chunk) receives key kperm(m) of its
-// 32-key sub-block, so that LDS row m is MFMA row m.
-template <int D, int ROWS, int THREADS, bool KEYS>
-__device__ __forceinline__ void load_tile(const Rows& r, int row0, uint4 (&reg)[ROWS * (D / 8) / THREADS]) {
-  constexpr int C8 = D / 8;
-#pragma unroll
-  for (int j = 0; j < ROWS * C8 / THREADS; ++j) {
-    const int cidx = threadIdx.x + THREADS * j;
-    const int m = cidx / C8;
-    const int src = KEYS ? ((m & ~31) | kperm(m & 31)) : m;
-    reg[j] = load16(r, row0 + src, (cidx % C8) * 16);
-  }
-}
-
-// Store such a tile row-major into LDS with a padded row stride of LROW elements.
-template <int D, int ROWS, int THREADS, int LROW>
-__device__ __forceinline__ void store_tile_padded(unsigned short* lds, const uint4 (&reg)[ROWS * (D / 8) / THREADS]) {
-  constexpr int C8 = D / 8;
-#pragma unroll
-  for (int j = 0; j < ROWS * C8 / THREADS; ++j) {
-    const int cidx = threadIdx.x + THREADS * j;
-    *reinterpret_cast<uint4*>(lds + (cidx / C8) * LROW + (cidx % C8) * 8) = reg[j];
-  }
-}
-
 // XOR swizzle of the 16-byte chunks of an UNPADDED row-major tile (row = D*2 bytes) that makes
 // both access patterns of a dual-use tile bank-conflict free: row reads (16 consecutive rows,
 // one chunk each) and transpose reads (4 consecutive rows, 64 contiguous bytes each).
@@ -443,16 +405,6 @@ struct TileCopy {
 template <int N>
 __device__ __forceinline__ void wait_loads() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-
-template <int D, int ROWS, int THREADS>
-__device__ __forceinline__ void store_tile_swizzled(unsigned short* lds, const uint4 (&reg)[ROWS * (D / 8) / THREADS]) {
-  constexpr int C8 = D / 8;
-#pragma unroll
-  for (int j = 0; j < ROWS * C8 / THREADS; ++j) {
-    const int cidx = threadIdx.x + THREADS * j;
-    *reinterpret_cast<uint4*>(lds + swz_off<D>(cidx / C8, cidx % C8)) = reg[j];
-  }
 }
 
 }  // namespace sba
