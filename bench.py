@@ -74,6 +74,10 @@ def main():
                          "heads, head_dim and scaling stay those of --workload)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--log-space", action="store_true", help="log2-sum carry instead of product carry")
+    ap.add_argument("--epilogue", default="none", choices=["none", "torch", "fused"],
+                    help="also form o + rem[..., None] * v, what callers do next (and differentiate through it): "
+                         "with PyTorch elementwise ops, or inside the kernels (sb_attn_varlen_fused). "
+                         "The headline metric is measured with 'none'.")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device copy (reference dispatch for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -83,7 +87,7 @@ def main():
 
     import torch
     from oracle import sb_oracle as orc
-    from stickbreaking_attention import _native, _ops, sb_attn, sb_attn_varlen
+    from stickbreaking_attention import _native, _ops, sb_attn, sb_attn_fused, sb_attn_varlen, sb_attn_varlen_fused
     if args.log_space:
         _ops.PRODUCT_SPACE = False
     lib = _native.load()
@@ -110,9 +114,17 @@ def main():
         q.requires_grad_(); k.requires_grad_(); v.requires_grad_()
 
     def attention():
+        if args.epilogue == "fused":
+            if fixed:
+                return sb_attn_fused(q, k, v), None
+            return sb_attn_varlen_fused(q, k, v, cu, max_len, zero_start=cfg["zero_start"]), None
         if fixed:
-            return sb_attn(q, k, v)
-        return sb_attn_varlen(q, k, v, cu, max_len, zero_start=cfg["zero_start"])
+            o, rem = sb_attn(q, k, v)
+        else:
+            o, rem = sb_attn_varlen(q, k, v, cu, max_len, zero_start=cfg["zero_start"])
+        if args.epilogue == "torch":
+            o = o + rem[..., None] * v
+        return o, rem
 
     def step():
         if backward:
@@ -185,7 +197,7 @@ def main():
         "config": {"workload": (f"{args.workload}: sb_attn fwd+bwd B={len(lengths)} H={H} T={T} d={d}, N(0,1)" if fixed else
                                f"{args.workload}: sb_attn_varlen {'fwd+bwd' if backward else 'fwd'} H={H} d={d} "
                                f"T={T} in {len(lengths)} documents (tests/golden/doc_lengths.json), N(0,1)*{cfg['scale']}"),
-                   "carry": "product" if _ops.PRODUCT_SPACE else "log2-sum", "sum_L2": sum(l * l for l in lengths)},
+                   "carry": "product" if _ops.PRODUCT_SPACE else "log2-sum", "epilogue": args.epilogue, "sum_L2": sum(l * l for l in lengths)},
         "fwd_ms": ms_fwd, "fwd_tflops": 4.0 * d * pairs / (ms_fwd * 1e-3) / 1e12,
         "frac_of_bf16_peak": total_flops / (ms_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
         "kernel_ms": dict(zip(names, kern_ms)),

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define SBA_VERSION 100
+#define SBA_VERSION 101
 
 /* error codes (negative returns) */
 #define SBA_E_NULL      (-1)  /* a required pointer is NULL                         */
@@ -59,6 +59,13 @@ extern "C" {
 #define SBA_PRODUCT_SPACE  4u   /* carry the stick as a running product instead of a
                                    running log2 sum (same results to ~1e-6, fewer
                                    transcendentals); must match between fwd and bwd       */
+#define SBA_FUSE_REMAINDER 16u  /* fold in what every upstream caller does next with the two
+                                   outputs (tests/test_varlen.py:101, tests/test_attn.py:64):
+                                   forward writes  o + rem[..., None] * v  into `o` (rem is
+                                   still written); backward takes `grad_o` as the gradient
+                                   of that sum and adds the terms it implies
+                                   (d rem += grad_o . v per row, dv += rem * grad_o).  No
+                                   upstream counterpart; must match between fwd and bwd    */
 
 /* A strided view over [batch, heads, tokens, head_dim]; the last dimension is contiguous.
  * Strides are in ELEMENTS.  For packed variable-length input batch == 1 and stride_b is
@@ -92,7 +99,8 @@ typedef struct sba_problem {
 /* Bytes of the schedule workspace (tile lists + status words) for this problem. */
 size_t sba_schedule_bytes(const sba_problem* p);
 
-/* Bytes of ONE carry table (fp32 [heads][ceil(max_doc_len/32)][batch*tokens]).  The forward
+/* Bytes of ONE carry table (fp32 [heads][ceil(max_doc_len/32) + 1][batch*tokens]; the last
+ * plane holds one value per row: rem, resp. the complete gradient of rem).  The forward
  * fills `stick_table`; the backward additionally needs a `grad_table` of the same size. */
 size_t sba_table_bytes(const sba_problem* p);
 

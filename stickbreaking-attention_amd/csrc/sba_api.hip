@@ -117,6 +117,8 @@ int fill_common(const sba_problem* p, const Sizes& sz, const void* schedule, KAr
   a->heads = p->heads;
   a->tokens = p->tokens;
   a->n_tt = sz.n_tt;
+  a->n_pl = sz.n_tt + 1;
+  a->fuse = (p->flags & SBA_FUSE_REMAINDER) ? 1 : 0;
   a->rows_total = sz.rows;
   a->inv_temp = p->inv_temp;
   a->c = p->inv_temp * 1.4426950408889634f;
@@ -225,7 +227,7 @@ size_t sba_table_bytes(const sba_problem* p) {
   Sizes sz;
   const bool fixed = p != nullptr && (p->flags & SBA_FIXED_LENGTH) != 0;
   if (check_problem(p, fixed, &sz)) return 0;
-  return (size_t)p->heads * (size_t)sz.n_tt * (size_t)sz.rows * sizeof(float);
+  return (size_t)p->heads * ((size_t)sz.n_tt + 1) * (size_t)sz.rows * sizeof(float);
 }
 
 int sba_build_schedule(const sba_problem* p, void* schedule, void* stream) {

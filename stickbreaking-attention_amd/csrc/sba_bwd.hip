@@ -151,10 +151,24 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
     qf[ks] = load_frag(qrows, qrow, 32 * ks + 16 * h);
     dof[ks] = load_frag(grows, qrow, 32 * ks + 16 * h);
   }
+  // d(rem) of this lane's row.  When the caller consumed o + rem * v, the gradient arriving for
+  // that sum also reaches rem, through the row's own value vector: d(rem) += do . v_row.
   float dr = 0.0f;
   if (a.grem.ptr != nullptr && qvalid) {
     const __bf16* grb = reinterpret_cast<const __bf16*>(a.grem.ptr) + t.batch * a.grem.sb + head * a.grem.sh + tok0 * a.grem.st;
     dr = (float)grb[(int64_t)qrow * a.grem.st];
+  }
+  if (a.fuse) {
+    float dot = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const bf16x8 vown = load_frag(vrows, qrow, 32 * ks + 16 * h);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dot = fmaf((float)dof[ks][e], (float)vown[e], dot);
+    }
+    float lo, hi;
+    both_halves(dot, lo, hi);
+    dr += lo + hi;
   }
 
   f32x16 dqacc[DB];
@@ -181,9 +195,11 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
       toff[u][db] = swz_off<D>(r, col >> 3) + (col & 7);
     }
   }
-  const int64_t tab0 = (int64_t)head * a.n_tt * a.rows_total + grow;
+  const int64_t tab0 = (int64_t)head * a.n_pl * a.rows_total + grow;
   const float* stick = a.stick + tab0;
   float* gtab = a.gtab + tab0;
+  // the dk/dv pass takes d(rem) from the last plane of the gradient table
+  if (qvalid && h == 0) gtab[(int64_t)a.n_tt * a.rows_total] = dr;
 
   // stick carries of the two sub-blocks of a tile (neutral where the sub-block is skipped)
   auto carries = [&](int kt, float (&ce)[2]) {
@@ -329,8 +345,6 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   const __bf16* kb = reinterpret_cast<const __bf16*>(a.k.ptr) + t.batch * a.k.sb + head * a.k.sh + tok0 * a.k.st;
   const __bf16* vb = reinterpret_cast<const __bf16*>(a.v.ptr) + t.batch * a.v.sb + head * a.v.sh + tok0 * a.v.st;
   const __bf16* gob = reinterpret_cast<const __bf16*>(a.go.ptr) + t.batch * a.go.sb + head * a.go.sh + tok0 * a.go.st;
-  const __bf16* grb = a.grem.ptr == nullptr ? nullptr
-      : reinterpret_cast<const __bf16*>(a.grem.ptr) + t.batch * a.grem.sb + head * a.grem.sh + tok0 * a.grem.st;
   const Rows qrows = make_rows(qb, a.q.st, t.doc_len);
   const Rows grows = make_rows(gob, a.go.st, t.doc_len);
   const Rows krows = make_rows(kb, a.k.st, t.doc_len);
@@ -359,28 +373,32 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     // reads are redirected to the document's last block so that they stay inside the tables
     // (which hold ceil(max_doc_len / 32) blocks per row), and their values are never used.
     const int tblock = min((BKV / 32) * kt + sb, (t.doc_len - 1) / 32);
-    const int64_t tab = (int64_t)head * a.n_tt * a.rows_total + (int64_t)t.batch * a.tokens + tok0 +
-                        (int64_t)tblock * a.rows_total;
+    const int64_t tab_row0 = (int64_t)head * a.n_pl * a.rows_total + (int64_t)t.batch * a.tokens + tok0;
+    const int64_t tab = tab_row0 + (int64_t)tblock * a.rows_total;
+    const int64_t tab_rowval = tab_row0 + (int64_t)a.n_tt * a.rows_total;   // per-row plane: rem (stick table), d(rem) (gradient table, written by the dq pass)
+    // Fused output o + rem * v: its gradient reaches v_j directly as rem_j * do_j.  The queries of
+    // step `sb` are this wave's own keys, so that term is dv = P^T dO with rem_j added on the
+    // diagonal of P (which is otherwise zero, or p_jj with attend_current), at no extra traffic.
+    float rem_own = 0.0f;
+    if (a.fuse && k0 + n < t.doc_len) rem_own = a.stick[tab_rowval + k0 + n];
     // Per-row carries of a step, branch-free: the address is clamped into the document and the
     // value replaced by the neutral element past its end (those rows have zero Q and dO).
-    const int64_t grem_st = grb != nullptr ? a.grem.st : 0;
-    const __bf16* grb_safe = grb != nullptr ? grb : reinterpret_cast<const __bf16*>(a.stick);
     // `request` only issues the loads; `settle` applies the end-of-document selection.  They are
     // kept apart so that nothing consumes (and therefore waits for) a loaded value until a
     // whole step after the request.
-    struct Raw { float e, g; unsigned short d; };   // d: grad_rem still as bf16 bits
+    struct Raw { float e, g, d; };
     auto request = [&](int step, Raw& r) {
       const int qrow = q_first + step * BQ + qr;
       const int qc = qrow < t.doc_len ? qrow : t.doc_len - 1;
       r.e = a.stick[tab + qc];
       r.g = a.gtab[tab + qc];
-      r.d = reinterpret_cast<const unsigned short*>(grb_safe)[(int64_t)qc * grem_st];
+      r.d = a.gtab[tab_rowval + qc];
     };
     auto settle = [&](int step, const Raw& r, float& ce, float& cc, float& d_r) {
       const bool ok = q_first + step * BQ + qr < t.doc_len;
       ce = ok ? r.e : (PROD ? 1.0f : 0.0f);
       cc = ok ? r.g : 0.0f;
-      d_r = (ok && grb != nullptr) ? __builtin_bit_cast(float, (unsigned)r.d << 16) : 0.0f;
+      d_r = ok ? r.d : 0.0f;
     };
     // The row-read offsets of this lane inside a tile (chunk 2*ks + h of row qr).
     int roff[KS];
@@ -447,6 +465,13 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
         else stick_weights<AC, PROD, false, true>(xc, a.c, k0, qrow, h, carry_e, p, bt, ends);
         pf[0] = pack8(p);
         pf[1] = pack8(p + 8);
+        if (DIAG && a.fuse && qw0 == k0) {
+          float pd[16];
+#pragma unroll
+          for (int j = 0; j < 16; ++j) pd[j] = p[j] + (16 * h + j == n ? rem_own : 0.0f);
+          pf[0] = pack8(pd);
+          pf[1] = pack8(pd + 8);
+        }
         grad_dz<PROD>(p, bt, dc, ends, h, carry_c, dr, zf);
       }
       stage(i & 1, pf, zf);

@@ -304,6 +304,45 @@ __device__ __forceinline__ void store_block32(unsigned short* scratch, const f32
   }
 }
 
+// Same, with a per-row multiple of another bf16 matrix added on the way out:
+//   out[row] = acc[row] * scale + rowscale(row) * addend[row]
+// (`rowscale(r)` = the fp32 factor of block row r, 0 <= r < 32, called once per 16-byte chunk).
+// The accumulators are rounded to bf16 once in the scratch, the sum is formed in fp32 and
+// rounded again: one rounding fewer than a caller adding the two bf16 tensors afterwards.
+template <int D, class RowScale>
+__device__ __forceinline__ void store_block32_axpy(unsigned short* scratch, const f32x16 (&acc)[D / 32], float scale,
+                                                   __bf16* out, int64_t stride_t, int row0, int limit, int lane,
+                                                   const __bf16* addend, int64_t addend_stride_t, RowScale rowscale) {
+  const int n = lane & 31, h = lane >> 5;
+  __bf16* sc = reinterpret_cast<__bf16*>(scratch);
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = 8 * (i >> 2) + 4 * h + (i & 3);
+      sc[row * D + 32 * db + n] = (__bf16)(acc[db][i] * scale);
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own LDS writes have landed
+  constexpr int C8 = D / 8;
+#pragma unroll
+  for (int j = 0; j < 32 * C8 / 64; ++j) {
+    const int cidx = lane + 64 * j;
+    const int row = cidx / C8, c8 = cidx % C8;
+    const bool ok = row0 + row < limit;
+    const float f = rowscale(row);
+    const bf16x8 mine = *reinterpret_cast<const bf16x8*>(scratch + row * D + c8 * 8);
+    bf16x8 other;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) other[e] = (__bf16)0.0f;
+    if (ok) other = *reinterpret_cast<const bf16x8*>(addend + (int64_t)(row0 + row) * addend_stride_t + c8 * 8);
+    float sum[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) sum[e] = fmaf(f, (float)other[e], (float)mine[e]);
+    if (ok) *reinterpret_cast<bf16x8*>(out + (int64_t)(row0 + row) * stride_t + c8 * 8) = pack8(sum);
+  }
+}
+
 // Is the 32-key sub-block starting at k0 entirely invisible / entirely visible to the 32
 // queries starting at qw0?
 template <bool AC>

@@ -93,7 +93,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
       voff[u][db] = swz_off<D>(r, col >> 3) + (col & 7);
     }
   }
-  float* stick = a.stick == nullptr ? nullptr : a.stick + (int64_t)head * a.n_tt * a.rows_total + grow;
+  float* stick = a.stick == nullptr ? nullptr : a.stick + (int64_t)head * a.n_pl * a.rows_total + grow;
 
   // One tile step; the ring slot is a compile-time constant so every LDS address is a fixed
   // register plus an immediate.
@@ -160,12 +160,20 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   }
 
   // epilogue: rem = what is left of the stick; o rows in the accumulator layout
+  const float r = PROD ? carry : fast_exp2(carry);
   if (h == 0 && qvalid) {
-    const float r = PROD ? carry : fast_exp2(carry);
     rb[(int64_t)qrow * a.rem.st] = (__bf16)r;
+    // rem in full precision for the backward of the fused output (last plane of the table)
+    if (stick != nullptr) stick[(int64_t)a.n_tt * a.rows_total] = r;
   }
   lds_barrier();   // every wave is done with the K/V tiles: their memory becomes the o staging area
-  store_block32<D>(smem + w * 32 * D, oacc, 1.0f, ob, a.o.st, qw0, t.doc_len, lane);
+  if (a.fuse) {
+    // what every caller computes next (upstream tests/test_varlen.py:101): o + rem * v
+    store_block32_axpy<D>(smem + w * 32 * D, oacc, 1.0f, ob, a.o.st, qw0, t.doc_len, lane, vb, a.v.st,
+                          [&](int row) { return __shfl(r, row, 64); });
+  } else {
+    store_block32<D>(smem + w * 32 * D, oacc, 1.0f, ob, a.o.st, qw0, t.doc_len, lane);
+  }
 }
 
 // Explicit instantiations: every (head_dim, attend_current, carry space) variant the launchers use.

@@ -17,6 +17,9 @@ struct KArgs {
   int heads;
   int tokens;                  // tokens per batch entry
   int n_tt;                    // table blocks per row = ceil(max_doc_len / 32)
+  int n_pl;                    // planes of a table = n_tt + 1; the last one holds per-row values
+                               // (stick table: rem in fp32; gradient table: the full d(rem))
+  int fuse;                    // the output is o + rem * v (and grad_o is the gradient of that)
   int64_t rows_total;          // batch * tokens
   float c;                     // inv_temp * log2(e)
   float inv_temp;

@@ -5,10 +5,10 @@ The two public operators have the names and signatures of upstream
 HIP behind the C ABI of ``include/sba.h``) and is loaded on first use.
 """
 from ._native import LIB_PATH as _LIB_PATH
-from .sb_attn import sb_attn
-from .sb_varlen import sb_attn_varlen
+from .sb_attn import sb_attn, sb_attn_fused
+from .sb_varlen import sb_attn_varlen, sb_attn_varlen_fused
 
-__all__ = ["sb_attn", "sb_attn_varlen", "library_path"]
+__all__ = ["sb_attn", "sb_attn_varlen", "sb_attn_fused", "sb_attn_varlen_fused", "library_path"]
 __version__ = "1.0.0"
 
 

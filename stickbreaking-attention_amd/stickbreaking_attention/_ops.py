@@ -54,7 +54,7 @@ def workspace_sizes(fixed: bool, batch: int, heads: int, tokens: int, n_docs: in
     n_kv = rows // _BKV + docs + 1
     words = _SCHED_HDR + 4 * (n_q + n_kv) + 5 * docs + 2
     n_tt = -(-max(1, max_doc_len if not fixed else tokens) // _BT)
-    return (4 * words + 255) & ~255, heads * n_tt * rows
+    return (4 * words + 255) & ~255, heads * (n_tt + 1) * rows
 
 
 def _prep(t: torch.Tensor, dpad: int, incoming_grad: bool = False) -> torch.Tensor:
@@ -78,9 +78,10 @@ def _aligned(t: torch.Tensor) -> torch.Tensor:
 
 
 def _problem(q: torch.Tensor, fixed: bool, cu_seqlens: Optional[torch.Tensor], max_doc_len: int,
-             inv_temp: float, attend_current: bool, product: bool):
+             inv_temp: float, attend_current: bool, product: bool, fused: bool):
     """The ``sba_problem`` of a launch plus the tensors whose pointers it holds."""
-    flags = (nat.FLAG_ATTEND_CURRENT if attend_current else 0) | (nat.FLAG_PRODUCT_SPACE if product else 0)
+    flags = ((nat.FLAG_ATTEND_CURRENT if attend_current else 0) | (nat.FLAG_PRODUCT_SPACE if product else 0) |
+             (nat.FLAG_FUSE_REMAINDER if fused else 0))
     if fixed:
         B, H, T, d = q.shape
         return nat.SbaProblem(nat.SBA_BF16, d, H, B, T, 0, T, flags | nat.FLAG_FIXED_LENGTH,
@@ -101,11 +102,11 @@ def _ptr(t: Optional[torch.Tensor]):
 # launchers: everything is allocated by the caller
 # ---------------------------------------------------------------------------------------------
 def _launch_fwd(fixed: bool, q, k, v, cu_seqlens, max_doc_len: int, logit_scale: float, attend_current: bool,
-                product: bool, o, rem, table, sched) -> None:
+                product: bool, fused: bool, o, rem, table, sched) -> None:
     nat.require_gpu(q)
     lib = nat.load()
     q, k, v = _aligned(q), _aligned(k), _aligned(v)
-    prob, _keep = _problem(q, fixed, cu_seqlens, max_doc_len, logit_scale, attend_current, product)
+    prob, _keep = _problem(q, fixed, cu_seqlens, max_doc_len, logit_scale, attend_current, product, fused)
     need, _ = workspace_sizes(fixed, prob.batch, prob.heads, prob.tokens, prob.n_docs, prob.max_doc_len)
     if sched.numel() * sched.element_size() < need:
         raise ValueError("schedule workspace too small")
@@ -121,11 +122,11 @@ def _launch_fwd(fixed: bool, q, k, v, cu_seqlens, max_doc_len: int, logit_scale:
 
 
 def _launch_bwd(fixed: bool, do, dr, q, k, v, cu_seqlens, max_doc_len: int, logit_scale: float,
-                attend_current: bool, product: bool, table, sched, gtab, dq, dk, dv) -> None:
+                attend_current: bool, product: bool, fused: bool, table, sched, gtab, dq, dk, dv) -> None:
     nat.require_gpu(q)
     lib = nat.load()
     q, k, v, do = _aligned(q), _aligned(k), _aligned(v), _aligned(do)
-    prob, _keep = _problem(q, fixed, cu_seqlens, max_doc_len, logit_scale, attend_current, product)
+    prob, _keep = _problem(q, fixed, cu_seqlens, max_doc_len, logit_scale, attend_current, product, fused)
     fn = lib.sba_attn_bwd if fixed else lib.sba_varlen_bwd
     drv = dr if dr is not None and dr.numel() else None
     with torch.cuda.device(q.device):
@@ -143,33 +144,34 @@ def _launch_bwd(fixed: bool, do, dr, q, k, v, cu_seqlens, max_doc_len: int, logi
 # written in place; `table` may be empty when no backward will follow.
 @custom_op("varlen_fwd", mutates_args={"o", "rem", "table", "sched"})
 def _compileable_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor,
-                         max_seqlens: int, logit_scale: float, attend_current: bool, product: bool,
+                         max_seqlens: int, logit_scale: float, attend_current: bool, product: bool, fused: bool,
                          o: torch.Tensor, rem: torch.Tensor, table: torch.Tensor, sched: torch.Tensor) -> None:
-    _launch_fwd(False, q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current, product, o, rem, table, sched)
+    _launch_fwd(False, q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current, product, fused,
+                o, rem, table, sched)
 
 
 @custom_op("varlen_bwd", mutates_args={"gtab", "dq", "dk", "dv"})
 def _compileable_backward(do: torch.Tensor, dr: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                           cu_seqlens: torch.Tensor, max_seqlens: int, logit_scale: float, attend_current: bool,
-                          product: bool, table: torch.Tensor, sched: torch.Tensor, gtab: torch.Tensor,
+                          product: bool, fused: bool, table: torch.Tensor, sched: torch.Tensor, gtab: torch.Tensor,
                           dq: torch.Tensor, dk: torch.Tensor, dv: torch.Tensor) -> None:
-    _launch_bwd(False, do, dr, q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current, product,
+    _launch_bwd(False, do, dr, q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current, product, fused,
                 table, sched, gtab, dq, dk, dv)
 
 
 @custom_op("attn_fwd", mutates_args={"o", "rem", "table", "sched"})
 def _compileable_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_scale: float, attend_current: bool,
-                     product: bool, o: torch.Tensor, rem: torch.Tensor, table: torch.Tensor,
+                     product: bool, fused: bool, o: torch.Tensor, rem: torch.Tensor, table: torch.Tensor,
                      sched: torch.Tensor) -> None:
-    _launch_fwd(True, q, k, v, None, q.shape[2], logit_scale, attend_current, product, o, rem, table, sched)
+    _launch_fwd(True, q, k, v, None, q.shape[2], logit_scale, attend_current, product, fused, o, rem, table, sched)
 
 
 @custom_op("attn_bwd", mutates_args={"gtab", "dq", "dk", "dv"})
 def _compileable_bwd(do: torch.Tensor, dr: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
-                     logit_scale: float, attend_current: bool, product: bool, table: torch.Tensor,
+                     logit_scale: float, attend_current: bool, product: bool, fused: bool, table: torch.Tensor,
                      sched: torch.Tensor, gtab: torch.Tensor, dq: torch.Tensor, dk: torch.Tensor,
                      dv: torch.Tensor) -> None:
-    _launch_bwd(True, do, dr, q, k, v, None, q.shape[2], logit_scale, attend_current, product,
+    _launch_bwd(True, do, dr, q, k, v, None, q.shape[2], logit_scale, attend_current, product, fused,
                 table, sched, gtab, dq, dk, dv)
 
 
@@ -187,9 +189,10 @@ def _check_cu(cu_seqlens: torch.Tensor, like: torch.Tensor) -> torch.Tensor:
 
 
 def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, attend_current: bool,
-            need_table: bool):
+                need_table: bool, fused: bool = False):
     """Returns (o, rem, state); ``state`` = (table, sched, cu_seqlens, max_doc_len, product) is what
-    the backward needs (upstream keeps its fp32 ``neg_log_acc`` there)."""
+    the backward needs (upstream keeps its fp32 ``neg_log_acc`` there).  With ``fused`` the first
+    output is ``o + rem[..., None] * v``."""
     nat.require_gpu(q)
     d = q.shape[-1]
     dpad = _padded_dim(d)
@@ -212,10 +215,11 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
     table = torch.empty(table_floats if need_table else 0, dtype=torch.float32, device=q.device)
     sched = torch.empty(sched_bytes, dtype=torch.uint8, device=q.device)
     if fixed:
-        _compileable_fwd(qp, kp, vp, float(inv_temp), bool(attend_current), product, o, rem, table, sched)
+        _compileable_fwd(qp, kp, vp, float(inv_temp), bool(attend_current), product, bool(fused),
+                         o, rem, table, sched)
     else:
         _compileable_forward(qp, kp, vp, cu, max_len, float(inv_temp), bool(attend_current), product,
-                             o, rem, table, sched)
+                             bool(fused), o, rem, table, sched)
         if VALIDATE and not torch.compiler.is_compiling():
             check_status(sched)
     if dpad != d or q.dtype != torch.bfloat16:
@@ -231,7 +235,9 @@ def check_status(sched: torch.Tensor) -> None:
         raise ValueError("sb_attn_varlen: " + nat.STATUS_MESSAGES.get(status, f"scheduler status {status}"))
 
 
-def run_backward(q, k, v, do, drem, fixed: bool, state, inv_temp: float, attend_current: bool, dkdv_dtype=None):
+def run_backward(q, k, v, do, drem, fixed: bool, state, inv_temp: float, attend_current: bool, dkdv_dtype=None,
+                 fused: bool = False):
+    """dq, dk, dv.  With ``fused``, ``do`` is the gradient of ``o + rem[..., None] * v``."""
     table, sched, cu, max_len, product = state
     d = q.shape[-1]
     dpad = _padded_dim(d)
@@ -246,11 +252,11 @@ def run_backward(q, k, v, do, drem, fixed: bool, state, inv_temp: float, attend_
     dq, dk, dv = torch.empty_like(qp), torch.empty_like(kp), torch.empty_like(vp)
     gtab = torch.empty_like(table)
     if fixed:
-        _compileable_bwd(dop, dremp, qp, kp, vp, float(inv_temp), bool(attend_current), product,
+        _compileable_bwd(dop, dremp, qp, kp, vp, float(inv_temp), bool(attend_current), product, bool(fused),
                          table, sched, gtab, dq, dk, dv)
     else:
         _compileable_backward(dop, dremp, qp, kp, vp, cu, max_len, float(inv_temp), bool(attend_current),
-                              product, table, sched, gtab, dq, dk, dv)
+                              product, bool(fused), table, sched, gtab, dq, dk, dv)
     if dpad != d or q.dtype != torch.bfloat16:
         dq = dq[..., :d].to(q.dtype)
         dk = dk[..., :d].to(k.dtype if dkdv_dtype is None else dkdv_dtype)

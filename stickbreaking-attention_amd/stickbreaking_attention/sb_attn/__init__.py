@@ -17,12 +17,13 @@ BWD_BLOCK_M = 128
 BWD_BLOCK_N = 64
 
 
-def _fwd(q, k, v, logit_scale, attend_current=False, no_grad=False):
-    return _ops.run_forward(q, k, v, True, None, None, logit_scale, attend_current, need_table=not no_grad)
+def _fwd(q, k, v, logit_scale, attend_current=False, no_grad=False, fused=False):
+    return _ops.run_forward(q, k, v, True, None, None, logit_scale, attend_current, need_table=not no_grad,
+                            fused=fused)
 
 
-def _bwd(do, dr, q, k, v, state, logit_scale, attend_current=False):
-    return _ops.run_backward(q, k, v, do, dr, True, state, logit_scale, attend_current)
+def _bwd(do, dr, q, k, v, state, logit_scale, attend_current=False, fused=False):
+    return _ops.run_backward(q, k, v, do, dr, True, state, logit_scale, attend_current, fused=fused)
 
 
 class StickBreakingAttention(torch.autograd.Function):
@@ -56,3 +57,35 @@ def sb_attn(q, k, v, inv_temp=None, zero_start=True, attend_current=False):
 
 def sb_attn_(q, k, v, inv_temp, attend_current):
     return StickBreakingAttention.apply(q, k, v, inv_temp, attend_current)
+
+
+class StickBreakingAttentionFused(torch.autograd.Function):
+    """``o + rem[..., None] * v`` in one piece (see ``sb_varlen.StickBreakingAttentionFused``)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, inv_temp, attend_current=False):
+        no_grad = not any(ctx.needs_input_grad[:3])
+        out, _rem, state = _fwd(q, k, v, logit_scale=inv_temp, attend_current=attend_current, no_grad=no_grad,
+                                fused=True)
+        table, sched, _cu, max_len, product = state
+        ctx.save_for_backward(q, k, v, table, sched)
+        ctx.logit_scale = inv_temp
+        ctx.max_seqlens = max_len
+        ctx.attend_current = attend_current
+        ctx.product = product
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, table, sched = ctx.saved_tensors
+        state = (table, sched, None, ctx.max_seqlens, ctx.product)
+        dq, dk, dv = _bwd(dout, None, q, k, v, state, ctx.logit_scale, ctx.attend_current, fused=True)
+        return dq, dk, dv, None, None
+
+
+def sb_attn_fused(q, k, v, inv_temp=None, zero_start=True, attend_current=False):
+    """Same arguments as ``sb_attn``; returns ``o + rem[..., None] * v`` (upstream
+    tests/test_attn.py:64) as one tensor."""
+    if inv_temp is None:
+        inv_temp = 1 / math.sqrt(q.size(-1))
+    return StickBreakingAttentionFused.apply(q, k, v, inv_temp, attend_current)

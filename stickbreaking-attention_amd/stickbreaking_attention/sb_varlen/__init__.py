@@ -17,15 +17,15 @@ BWD_BLOCK_M = 128
 BWD_BLOCK_N = 64
 
 
-def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=False, no_grad=False):
+def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=False, no_grad=False, fused=False):
     """Host launcher of the forward; returns (o, rem, state) where ``state`` is what the
     backward needs (carry table, schedule, ...) -- upstream returns its fp32 ``neg_log_acc`` there."""
     return _ops.run_forward(q, k, v, False, cu_seqlens, max_seqlens, logit_scale, attend_current,
-                        need_table=not no_grad)
+                            need_table=not no_grad, fused=fused)
 
 
-def varlen_bwd(do, dr, q, k, v, state, logit_scale, attend_current=False):
-    return _ops.run_backward(q, k, v, do, dr, False, state, logit_scale, attend_current)
+def varlen_bwd(do, dr, q, k, v, state, logit_scale, attend_current=False, fused=False):
+    return _ops.run_backward(q, k, v, do, dr, False, state, logit_scale, attend_current, fused=fused)
 
 
 class StickBreakingAttention(torch.autograd.Function):
@@ -65,3 +65,40 @@ def sb_attn_varlen(q, k, v, cu_seqlens, max_seqlens=None, inv_temp=None, zero_st
 
 def sb_attn_varlen_(q, k, v, inv_temp, cu_seqlens, max_seqlens, attend_current):
     return StickBreakingAttention.apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current)
+
+
+class StickBreakingAttentionFused(torch.autograd.Function):
+    """``o + rem[..., None] * v`` in one piece: the sum is formed where ``o`` leaves the forward
+    kernel, and its gradient's two extra terms inside the backward kernels."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current):
+        no_grad = not any(ctx.needs_input_grad[:3])
+        out, _rem, state = varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale=inv_temp,
+                                      attend_current=attend_current, no_grad=no_grad, fused=True)
+        table, sched, cu, max_len, product = state
+        ctx.save_for_backward(q, k, v, table, sched, cu)
+        ctx.logit_scale = inv_temp
+        ctx.max_seqlens = max_len
+        ctx.attend_current = attend_current
+        ctx.product = product
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, table, sched, cu = ctx.saved_tensors
+        state = (table, sched, cu, ctx.max_seqlens, ctx.product)
+        dq, dk, dv = varlen_bwd(dout, None, q, k, v, state, ctx.logit_scale, ctx.attend_current, fused=True)
+        return dq, dk, dv, None, None, None, None
+
+
+def sb_attn_varlen_fused(q, k, v, cu_seqlens, max_seqlens=None, inv_temp=None, zero_start=True, attend_current=False):
+    """Same arguments as ``sb_attn_varlen``; returns the single tensor every upstream caller forms
+    from its two outputs, ``o + rem[..., None] * v`` (upstream tests/test_varlen.py:101), without
+    the extra passes over ``o`` and ``v`` in forward and backward."""
+    if zero_start:
+        assert cu_seqlens[0] == 0
+        cu_seqlens = cu_seqlens[1:]
+    if inv_temp is None:
+        inv_temp = 1 / math.sqrt(q.size(-1))
+    return StickBreakingAttentionFused.apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current)

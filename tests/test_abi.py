@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for s in syms:
         assert hasattr(lib, s), f"{s} declared in include/sba.h but not exported"
     assert sorted(nat.EXPORTS) == syms
-    assert lib.sba_version() == 100
+    assert lib.sba_version() == 101
 
 
 def problem(**kw):
@@ -41,10 +41,11 @@ def test_workspace_sizes():
     sched = lib.sba_schedule_bytes(ctypes.byref(p))
     # two tile lists (16 B per tile): query tiles and key tiles, each bounded by tokens/128 + docs
     assert 16 * (128 + 8 + 128 + 8) <= sched <= 16 * (128 + 128 + 32) + 1024
-    assert lib.sba_table_bytes(ctypes.byref(p)) == 32 * 128 * 16384 * 4
+    # one plane per 32-key block of the longest document plus one plane of per-row values
+    assert lib.sba_table_bytes(ctypes.byref(p)) == 32 * (128 + 1) * 16384 * 4
     pf = problem(batch=4, heads=16, tokens=2048, n_docs=0, max_doc_len=2048, head_dim=64,
                  flags=nat.FLAG_FIXED_LENGTH, cu_seqlens=None)
-    assert lib.sba_table_bytes(ctypes.byref(pf)) == 16 * 64 * 4 * 2048 * 4
+    assert lib.sba_table_bytes(ctypes.byref(pf)) == 16 * (64 + 1) * 4 * 2048 * 4
 
 
 @pytest.mark.parametrize("kw,code", [
