@@ -269,6 +269,13 @@ __device__ __forceinline__ void stick_weights_fwd(const f32x16& x, float c, int 
     p[4 * g + 2] = a3 - a2;
     p[4 * g + 3] = before - a3;
   }
+  if (BAND) {
+    // A masked key leaves the stick as it was, but s * (1/u) * u only equals s to rounding:
+    // make its weight exactly zero so that nothing of a later token reaches this row.
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      if (!(i < lim)) p[i] = 0.0f;
+  }
   carry *= lo * hi;
 }
 

@@ -276,6 +276,26 @@ def test_backward_is_deterministic():
 # ---------------------------------------------------------------------------------------------
 # API behaviour
 # ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("ac", [False, True])
+def test_later_tokens_cannot_reach_earlier_rows(ac):
+    """Exact causality: replacing the keys and values of every token after position c leaves the
+    rows up to c bit-identical (a masked weight must be exactly zero, not zero to rounding)."""
+    from stickbreaking_attention import sb_attn_varlen
+    lengths, c = [333, 180], 201
+    q, k, v, _ = orc.make_inputs((2, sum(lengths), 128), 15)
+    cu = cu_from_lengths(lengths, device=DEV)
+    k2, v2 = k.clone(), v.clone()
+    k2[:, c + 1:lengths[0]] = 3.0
+    v2[:, c + 1:lengths[0]] = -50.0
+    with torch.no_grad():
+        o1, r1 = sb_attn_varlen(q.to(DEV), k.to(DEV), v.to(DEV), cu, max(lengths), zero_start=False, attend_current=ac)
+        o2, r2 = sb_attn_varlen(q.to(DEV), k2.to(DEV), v2.to(DEV), cu, max(lengths), zero_start=False, attend_current=ac)
+    torch.cuda.synchronize()
+    assert torch.equal(o1[:, :c + 1], o2[:, :c + 1]) and torch.equal(r1[:, :c + 1], r2[:, :c + 1])
+    assert torch.equal(o1[:, lengths[0]:], o2[:, lengths[0]:])
+    assert not torch.equal(o1[:, c + 2:lengths[0]], o2[:, c + 2:lengths[0]])
+
+
 def test_zero_start_int64_and_inv_temp():
     lengths = [100, 260, 77]
     q, k, v, do = orc.make_inputs((2, sum(lengths), 64), 21)
