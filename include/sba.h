@@ -134,6 +134,23 @@ int sba_attn_fwd(const sba_problem* p, const void* schedule,
                  const sba_view* o, const sba_view* rem,
                  float* stick_table, void* stream);
 
+/* Debug variants that additionally write the attention weights A[i,j] (fp32, before the bf16
+ * rounding that feeds A.V) of every causal in-document pair into `weights`, a dense
+ * [batch][heads][tokens][tokens] array (row = query token, column = key token; packed
+ * variable-length input: batch == 1 and both indices are positions in the packed sequence).
+ * Elements outside the causal triangle of a document are not written: clear the array first.
+ * Replaces upstream's `return_attention=True` launches (sb_varlen_fwd.py:195-202, :421-425;
+ * sb_attn/sb_fwd.py:147-151).  Quadratic memory; a separate, slower kernel instantiation. */
+int sba_varlen_fwd_weights(const sba_problem* p, const void* schedule,
+                           const sba_view* q, const sba_view* k, const sba_view* v,
+                           const sba_view* o, const sba_view* rem,
+                           float* stick_table, float* weights, void* stream);
+
+int sba_attn_fwd_weights(const sba_problem* p, const void* schedule,
+                         const sba_view* q, const sba_view* k, const sba_view* v,
+                         const sba_view* o, const sba_view* rem,
+                         float* stick_table, float* weights, void* stream);
+
 /* ---- backward --------------------------------------------------------------------------- */
 
 /* dq, dk, dv for every token (zero for tokens that belong to no document).  `stick_table` is the

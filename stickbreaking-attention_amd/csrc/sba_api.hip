@@ -126,7 +126,7 @@ int fill_common(const sba_problem* p, const Sizes& sz, const void* schedule, KAr
 }
 
 int forward(const sba_problem* p, bool fixed, const void* schedule, const sba_view* q, const sba_view* k,
-            const sba_view* v, const sba_view* o, const sba_view* rem, float* stick, void* stream) {
+            const sba_view* v, const sba_view* o, const sba_view* rem, float* stick, float* weights, void* stream) {
   Sizes sz;
   int e = check_problem(p, fixed, &sz);
   if (e) return e;
@@ -139,12 +139,13 @@ int forward(const sba_problem* p, bool fixed, const void* schedule, const sba_vi
   if ((e = fill_common(p, sz, schedule, &a))) return e;
   a.q = to_view(q); a.k = to_view(k); a.v = to_view(v); a.o = to_view(o); a.rem = to_view(rem);
   a.stick = stick;
+  a.weights = weights;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   hipError_t he = hipSuccess;
   if (sz.n_docs > 0) {
     Timer tm(0, s);
     he = launch_fwd(a, p->head_dim, (p->flags & SBA_ATTEND_CURRENT) != 0,
-                    (p->flags & SBA_PRODUCT_SPACE) != 0, sz.n_q_max, s);
+                    (p->flags & SBA_PRODUCT_SPACE) != 0, weights != nullptr, sz.n_q_max, s);
   }
   if (he != hipSuccess || fixed) return (int)he;
   ZeroArgs z;
@@ -252,13 +253,27 @@ int sba_build_schedule(const sba_problem* p, void* schedule, void* stream) {
 int sba_varlen_fwd(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
                    const sba_view* v, const sba_view* o, const sba_view* rem, float* stick_table,
                    void* stream) {
-  return forward(p, false, schedule, q, k, v, o, rem, stick_table, stream);
+  return forward(p, false, schedule, q, k, v, o, rem, stick_table, nullptr, stream);
 }
 
 int sba_attn_fwd(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
                  const sba_view* v, const sba_view* o, const sba_view* rem, float* stick_table,
                  void* stream) {
-  return forward(p, true, schedule, q, k, v, o, rem, stick_table, stream);
+  return forward(p, true, schedule, q, k, v, o, rem, stick_table, nullptr, stream);
+}
+
+int sba_varlen_fwd_weights(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
+                           const sba_view* v, const sba_view* o, const sba_view* rem, float* stick_table,
+                           float* weights, void* stream) {
+  if (weights == nullptr) return SBA_E_NULL;
+  return forward(p, false, schedule, q, k, v, o, rem, stick_table, weights, stream);
+}
+
+int sba_attn_fwd_weights(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
+                         const sba_view* v, const sba_view* o, const sba_view* rem, float* stick_table,
+                         float* weights, void* stream) {
+  if (weights == nullptr) return SBA_E_NULL;
+  return forward(p, true, schedule, q, k, v, o, rem, stick_table, weights, stream);
 }
 
 int sba_varlen_bwd(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,

@@ -10,7 +10,11 @@
 
 namespace sba {
 
-template <int D, bool AC, bool PROD>
+// WOUT: also write the attention weights (fp32, before their bf16 rounding) into a dense
+// [tokens x tokens] matrix per (batch, head) -- upstream's `return_attention` debug output
+// (sb_varlen_fwd.py:195-202).  A separate instantiation, so the production kernel carries none
+// of it.
+template <int D, bool AC, bool PROD, bool WOUT>
 __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   constexpr int KS = D / 16;     // contraction steps of K.Q^T
   constexpr int DB = D / 32;     // 32-wide output column blocks of P.V
@@ -133,6 +137,17 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
       if (sub_full<AC>(k0, qw0)) stick_weights<AC, PROD, false, false>(x, a.c, k0, qrow, h, carry, p, unused);
       else stick_weights<AC, PROD, true, false>(x, a.c, k0, qrow, h, carry, p, unused);
     }
+    if constexpr (WOUT) {
+      // this lane: query qrow, keys k0 + 16*h + i; masked positions already hold 0
+      if (qvalid) {
+        float* wrow = a.weights + (((int64_t)t.batch * a.heads + head) * a.tokens + tok0 + qrow) * a.tokens + tok0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = k0 + 16 * h + i;
+          if (key < t.doc_len) wrow[key] = p[i];
+        }
+      }
+    }
     // P as the A operand of O = P.V: slot s of step tt is key 16*h + 8*tt + s, which the
     // permuted tile keeps in LDS row 16*tt + 8*(s/4) + 4*h + s%4.
     bf16x8 vfr[2][DB];
@@ -177,31 +192,43 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
 }
 
 // Explicit instantiations: every (head_dim, attend_current, carry space) variant the launchers use.
-template __global__ void fwd_kernel<64, false, false>(const KArgs);
-template __global__ void fwd_kernel<64, false, true>(const KArgs);
-template __global__ void fwd_kernel<64, true, false>(const KArgs);
-template __global__ void fwd_kernel<64, true, true>(const KArgs);
-template __global__ void fwd_kernel<128, false, false>(const KArgs);
-template __global__ void fwd_kernel<128, false, true>(const KArgs);
-template __global__ void fwd_kernel<128, true, false>(const KArgs);
-template __global__ void fwd_kernel<128, true, true>(const KArgs);
+template __global__ void fwd_kernel<64, false, false, false>(const KArgs);
+template __global__ void fwd_kernel<64, false, false, true>(const KArgs);
+template __global__ void fwd_kernel<64, false, true, false>(const KArgs);
+template __global__ void fwd_kernel<64, false, true, true>(const KArgs);
+template __global__ void fwd_kernel<64, true, false, false>(const KArgs);
+template __global__ void fwd_kernel<64, true, false, true>(const KArgs);
+template __global__ void fwd_kernel<64, true, true, false>(const KArgs);
+template __global__ void fwd_kernel<64, true, true, true>(const KArgs);
+template __global__ void fwd_kernel<128, false, false, false>(const KArgs);
+template __global__ void fwd_kernel<128, false, false, true>(const KArgs);
+template __global__ void fwd_kernel<128, false, true, false>(const KArgs);
+template __global__ void fwd_kernel<128, false, true, true>(const KArgs);
+template __global__ void fwd_kernel<128, true, false, false>(const KArgs);
+template __global__ void fwd_kernel<128, true, false, true>(const KArgs);
+template __global__ void fwd_kernel<128, true, true, false>(const KArgs);
+template __global__ void fwd_kernel<128, true, true, true>(const KArgs);
 
-template <int D>
+template <int D, bool WOUT>
 static hipError_t launch_fwd_d(const KArgs& a, bool ac, bool prod, int n_q_max, hipStream_t s) {
   const dim3 grid((unsigned)n_q_max * (unsigned)a.heads), block(NT);
   if (ac) {
-    if (prod) hipLaunchKernelGGL((fwd_kernel<D, true, true>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((fwd_kernel<D, true, false>), grid, block, 0, s, a);
+    if (prod) hipLaunchKernelGGL((fwd_kernel<D, true, true, WOUT>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((fwd_kernel<D, true, false, WOUT>), grid, block, 0, s, a);
   } else {
-    if (prod) hipLaunchKernelGGL((fwd_kernel<D, false, true>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((fwd_kernel<D, false, false>), grid, block, 0, s, a);
+    if (prod) hipLaunchKernelGGL((fwd_kernel<D, false, true, WOUT>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((fwd_kernel<D, false, false, WOUT>), grid, block, 0, s, a);
   }
   return hipGetLastError();
 }
 
-hipError_t launch_fwd(const KArgs& a, int head_dim, bool ac, bool prod, int n_q_max, hipStream_t s) {
-  if (head_dim == 128) return launch_fwd_d<128>(a, ac, prod, n_q_max, s);
-  return launch_fwd_d<64>(a, ac, prod, n_q_max, s);
+hipError_t launch_fwd(const KArgs& a, int head_dim, bool ac, bool prod, bool weights, int n_q_max, hipStream_t s) {
+  if (weights) {
+    if (head_dim == 128) return launch_fwd_d<128, true>(a, ac, prod, n_q_max, s);
+    return launch_fwd_d<64, true>(a, ac, prod, n_q_max, s);
+  }
+  if (head_dim == 128) return launch_fwd_d<128, false>(a, ac, prod, n_q_max, s);
+  return launch_fwd_d<64, false>(a, ac, prod, n_q_max, s);
 }
 
 }  // namespace sba

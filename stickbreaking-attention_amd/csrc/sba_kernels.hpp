@@ -14,6 +14,8 @@ struct KArgs {
   int kv_list_off;             // int32 offset of the KV tile list inside `sched`
   float* stick;                // carry table written by the forward (may be null in fwd)
   float* gtab;                 // gradient prefix table (backward scratch)
+  float* weights;              // forward, debug variant only: dense attention weights
+                               // [batch][heads][tokens][tokens] (row = query token, column = key token)
   int heads;
   int tokens;                  // tokens per batch entry
   int n_tt;                    // table blocks per row = ceil(max_doc_len / 32)
@@ -46,8 +48,8 @@ struct ZeroArgs {
 
 hipError_t launch_schedule(const SchedArgs& a, hipStream_t s);
 hipError_t launch_zero_tail(const ZeroArgs& a, hipStream_t s);
-hipError_t launch_fwd(const KArgs& a, int head_dim, bool attend_current, bool product, int n_q_max,
-                      hipStream_t s);
+hipError_t launch_fwd(const KArgs& a, int head_dim, bool attend_current, bool product, bool weights,
+                      int n_q_max, hipStream_t s);
 hipError_t launch_bwd_dq(const KArgs& a, int head_dim, bool attend_current, bool product, int n_q_max,
                          hipStream_t s);
 hipError_t launch_bwd_dkdv(const KArgs& a, int head_dim, bool attend_current, bool product,

@@ -45,7 +45,7 @@ class SbaProblem(ctypes.Structure):
 EXPORTS = (
     "sba_version", "sba_error_string", "sba_schedule_bytes", "sba_table_bytes", "sba_build_schedule",
     "sba_varlen_fwd", "sba_varlen_bwd", "sba_attn_fwd", "sba_attn_bwd", "sba_set_timing",
-    "sba_last_kernel_ms",
+    "sba_last_kernel_ms", "sba_varlen_fwd_weights", "sba_attn_fwd_weights",
 )
 
 _lib = None
@@ -79,6 +79,10 @@ def load():
             f = getattr(lib, name)
             f.restype = ctypes.c_int
             f.argtypes = [P, vp, V, V, V, V, V, vp, vp]
+        for name in ("sba_varlen_fwd_weights", "sba_attn_fwd_weights"):
+            f = getattr(lib, name)
+            f.restype = ctypes.c_int
+            f.argtypes = [P, vp, V, V, V, V, V, vp, vp, vp]
         for name in ("sba_varlen_bwd", "sba_attn_bwd"):
             f = getattr(lib, name)
             f.restype = ctypes.c_int

@@ -102,7 +102,7 @@ def _ptr(t: Optional[torch.Tensor]):
 # launchers: everything is allocated by the caller
 # ---------------------------------------------------------------------------------------------
 def _launch_fwd(fixed: bool, q, k, v, cu_seqlens, max_doc_len: int, logit_scale: float, attend_current: bool,
-                product: bool, fused: bool, o, rem, table, sched) -> None:
+                product: bool, fused: bool, o, rem, table, sched, weights=None) -> None:
     nat.require_gpu(q)
     lib = nat.load()
     q, k, v = _aligned(q), _aligned(k), _aligned(v)
@@ -110,15 +110,17 @@ def _launch_fwd(fixed: bool, q, k, v, cu_seqlens, max_doc_len: int, logit_scale:
     need, _ = workspace_sizes(fixed, prob.batch, prob.heads, prob.tokens, prob.n_docs, prob.max_doc_len)
     if sched.numel() * sched.element_size() < need:
         raise ValueError("schedule workspace too small")
-    fn = lib.sba_attn_fwd if fixed else lib.sba_varlen_fwd
+    name = ("sba_attn_fwd" if fixed else "sba_varlen_fwd") + ("_weights" if weights is not None else "")
+    fn = getattr(lib, name)
+    extra = () if weights is None else (weights.data_ptr(),)
     with torch.cuda.device(q.device):
         stream = nat.stream_ptr(q.device)
         nat.check(lib.sba_build_schedule(ctypes.byref(prob), sched.data_ptr(), stream), "sba_build_schedule")
         code = fn(ctypes.byref(prob), sched.data_ptr(),
                   ctypes.byref(nat.view4(q, fixed)), ctypes.byref(nat.view4(k, fixed)),
                   ctypes.byref(nat.view4(v, fixed)), ctypes.byref(nat.view4(o, fixed)),
-                  ctypes.byref(nat.view4(rem, fixed, per_row=True)), _ptr(table), stream)
-    nat.check(code, "sba_attn_fwd" if fixed else "sba_varlen_fwd")
+                  ctypes.byref(nat.view4(rem, fixed, per_row=True)), _ptr(table), *extra, stream)
+    nat.check(code, name)
 
 
 def _launch_bwd(fixed: bool, do, dr, q, k, v, cu_seqlens, max_doc_len: int, logit_scale: float,
@@ -189,10 +191,12 @@ def _check_cu(cu_seqlens: torch.Tensor, like: torch.Tensor) -> torch.Tensor:
 
 
 def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, attend_current: bool,
-                need_table: bool, fused: bool = False):
+                need_table: bool, fused: bool = False, return_attention: bool = False):
     """Returns (o, rem, state); ``state`` = (table, sched, cu_seqlens, max_doc_len, product) is what
     the backward needs (upstream keeps its fp32 ``neg_log_acc`` there).  With ``fused`` the first
-    output is ``o + rem[..., None] * v``."""
+    output is ``o + rem[..., None] * v``.  With ``return_attention`` a fourth value follows: the
+    dense fp32 attention weights ``[(B,) H, T, T]`` (upstream sb_varlen_fwd.py:421-425,
+    sb_fwd.py:147-151; eager mode only, quadratic memory)."""
     nat.require_gpu(q)
     d = q.shape[-1]
     dpad = _padded_dim(d)
@@ -214,7 +218,11 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
     rem = torch.empty_like(qp[..., 0])
     table = torch.empty(table_floats if need_table else 0, dtype=torch.float32, device=q.device)
     sched = torch.empty(sched_bytes, dtype=torch.uint8, device=q.device)
-    if fixed:
+    if return_attention:
+        weights = torch.zeros(qp.shape[:-1] + (T,), dtype=torch.float32, device=q.device)
+        _launch_fwd(fixed, qp, kp, vp, cu, max_len, float(inv_temp), bool(attend_current), product, bool(fused),
+                    o, rem, table, sched, weights=weights)
+    elif fixed:
         _compileable_fwd(qp, kp, vp, float(inv_temp), bool(attend_current), product, bool(fused),
                          o, rem, table, sched)
     else:
@@ -225,7 +233,8 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
     if dpad != d or q.dtype != torch.bfloat16:
         o = o[..., :d].to(q.dtype)
         rem = rem.to(q.dtype)
-    return o, rem, (table, sched, cu, max_len, product)
+    state = (table, sched, cu, max_len, product)
+    return (o, rem, state, weights) if return_attention else (o, rem, state)
 
 
 def check_status(sched: torch.Tensor) -> None:

@@ -17,9 +17,10 @@ BWD_BLOCK_M = 128
 BWD_BLOCK_N = 64
 
 
-def _fwd(q, k, v, logit_scale, attend_current=False, no_grad=False, fused=False):
+def _fwd(q, k, v, logit_scale, attend_current=False, no_grad=False, return_attention=False, fused=False):
+    """(o, rem, state[, W [batch, heads, tokens, tokens]]) -- upstream sb_attn/sb_fwd.py:139-174."""
     return _ops.run_forward(q, k, v, True, None, None, logit_scale, attend_current, need_table=not no_grad,
-                            fused=fused)
+                            fused=fused, return_attention=return_attention)
 
 
 def _bwd(do, dr, q, k, v, state, logit_scale, attend_current=False, fused=False):

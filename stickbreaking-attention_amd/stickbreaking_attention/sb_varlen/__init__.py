@@ -17,11 +17,14 @@ BWD_BLOCK_M = 128
 BWD_BLOCK_N = 64
 
 
-def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=False, no_grad=False, fused=False):
+def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=False, no_grad=False,
+               return_attention=False, fused=False):
     """Host launcher of the forward; returns (o, rem, state) where ``state`` is what the
-    backward needs (carry table, schedule, ...) -- upstream returns its fp32 ``neg_log_acc`` there."""
+    backward needs (carry table, schedule, ...) -- upstream returns its fp32 ``neg_log_acc`` there --
+    and, with ``return_attention``, the dense fp32 weights ``W [heads, tokens, tokens]`` as a
+    fourth value (upstream sb_varlen_fwd.py:413-451)."""
     return _ops.run_forward(q, k, v, False, cu_seqlens, max_seqlens, logit_scale, attend_current,
-                            need_table=not no_grad, fused=fused)
+                            need_table=not no_grad, fused=fused, return_attention=return_attention)
 
 
 def varlen_bwd(do, dr, q, k, v, state, logit_scale, attend_current=False, fused=False):
