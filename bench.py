@@ -24,7 +24,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X published dense bf16 MFMA peak
 # same counter reads for the 256 MiB device copy of --calibrate-copy (FETCH_SIZE x2.0,
 # WRITE_SIZE x1.0).  Counters cannot be read from inside the process, so these are recorded
 # constants; other workloads report null.
-MEASURED_TRAFFIC_BYTES = {"c3": {"fwd_kernel": 1.136e9, "bwd_dq_kernel": 1.090e9, "bwd_dkdv_kernel": 1.201e9}}
+MEASURED_TRAFFIC_BYTES = {"c3": {"fwd_kernel": 1.164e9, "bwd_dq_kernel": 1.111e9, "bwd_dkdv_kernel": 1.202e9}}
 
 
 def workload(name):
