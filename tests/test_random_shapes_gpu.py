@@ -1,0 +1,68 @@
+"""Seeded random sweep over the argument space of the variable-length operators: document
+lengths around the tile edges (32, 64, 128 and their neighbours), empty documents, tail tokens
+outside every document, 1-3 heads, both head dims, strict / attend_current, int32 / int64
+cu_seqlens with and without the leading zero, over-stated or missing max_seqlens, with and
+without a gradient for rem, two-output and fused forms.  Each case is compared with the fp32
+oracle at the usual tolerance (max-abs 2e-2 plus the bf16 half-ulp of large values)."""
+import os
+import random
+
+import pytest
+import torch
+
+from oracle import sb_oracle as orc
+from tests.helpers import assert_close, cu_from_lengths, oracle_varlen
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+EDGES = [1, 2, 31, 32, 33, 63, 64, 65, 95, 96, 97, 127, 128, 129, 159, 160, 191, 192, 193, 255, 256, 257, 383, 384,
+         385, 511, 512, 513, 640, 700, 1023, 1025]
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from stickbreaking_attention import _native as nat
+    assert os.path.exists(nat.LIB_PATH), "libsba.so must be built before the GPU tests run"
+    nat.load()
+
+
+@pytest.mark.parametrize("case", range(24))
+def test_random_case(case):
+    from stickbreaking_attention import sb_attn_varlen, sb_attn_varlen_fused
+    rng = random.Random(9000 + case)
+    lengths = [rng.choice(EDGES) if rng.random() < 0.7 else rng.randint(1, 900) for _ in range(rng.choice([1, 2, 3, 5, 9]))]
+    if rng.random() < 0.25:
+        lengths.insert(rng.randrange(len(lengths) + 1), 0)
+    tail = rng.choice([0, 0, 1, 7, 40])
+    T, n_tok = sum(lengths) + tail, sum(lengths)
+    H, d, ac = rng.choice([1, 2, 3]), rng.choice([64, 128]), rng.random() < 0.5
+    fused = rng.random() < 0.4
+    q, k, v, do = orc.make_inputs((H, T, d), 1000 + case, dist=rng.choice(["normal", "upstream"]))
+    zero_start = rng.random() < 0.5
+    cu = cu_from_lengths(lengths, leading_zero=zero_start, dtype=rng.choice([torch.int32, torch.int64]), device=DEV)
+    max_seqlens = rng.choice([max(lengths), max(lengths) + 17, T, None])
+    drem = None
+    if not fused and rng.random() < 0.5:
+        drem = torch.randn((H, T), generator=torch.Generator().manual_seed(case)).to(torch.bfloat16)
+    print(f"lengths={lengths} tail={tail} H={H} d={d} ac={ac} fused={fused} zero_start={zero_start} "
+          f"cu={cu.dtype} max_seqlens={max_seqlens} drem={drem is not None}", flush=True)
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    if fused:
+        out = sb_attn_varlen_fused(qg, kg, vg, cu, max_seqlens, zero_start=zero_start, attend_current=ac)
+        got = (out.detach(),) + torch.autograd.grad(out, (qg, kg, vg), do.to(DEV))
+        vf, df = v.float(), do.float()
+        inside = (torch.arange(T) < n_tok)[None, :, None]
+        o, rem, dq, dk, dv = oracle_varlen(q, k, v, do, lengths, ac, drem=(df * vf).sum(-1))
+        ref = (o + rem[..., None] * vf * inside, dq, dk, dv + rem[..., None] * df * inside)
+        names = ("out", "dq", "dk", "dv")
+    else:
+        o, rem = sb_attn_varlen(qg, kg, vg, cu, max_seqlens, zero_start=zero_start, attend_current=ac)
+        outs, grads = ((o,), (do.to(DEV),)) if drem is None else ((o, rem), (do.to(DEV), drem.to(DEV)))
+        got = (o.detach(), rem.detach()) + torch.autograd.grad(outs, (qg, kg, vg), grads)
+        ref = oracle_varlen(q, k, v, do, lengths, ac, drem=drem)
+        names = ("o", "rem", "dq", "dk", "dv")
+    torch.cuda.synchronize()
+    for name, g, r in zip(names, got, ref):
+        assert_close(name, g, r)
