@@ -296,6 +296,15 @@ def test_later_tokens_cannot_reach_earlier_rows(ac):
     assert not torch.equal(o1[:, c + 2:lengths[0]], o2[:, c + 2:lengths[0]])
 
 
+@pytest.mark.parametrize("lengths", [[4] * 4096, [3] * 5000 + [700], [1] * 2000 + [129] * 20],
+                         ids=["4096x4", "5000x3+700", "2000x1+20x129"])
+def test_thousands_of_tiny_documents(lengths):
+    """The device scheduler with thousands of documents, below and above the number it still
+    ranks by length."""
+    q, k, v, do = orc.make_inputs((2, sum(lengths), 64), 3)
+    check_all(run_varlen(q, k, v, do, lengths), oracle_varlen(q, k, v, do, lengths))
+
+
 def test_zero_start_int64_and_inv_temp():
     lengths = [100, 260, 77]
     q, k, v, do = orc.make_inputs((2, sum(lengths), 64), 21)
