@@ -47,6 +47,58 @@ __global__ void __launch_bounds__(256, 4) mix_kernel(float* out, int reps) {
   out[blockIdx.x * 256 + threadIdx.x] = sum;
 }
 
+// Same question at a coarser grain: G MFMAs back to back (into four accumulators) followed by
+// G * VF independent FMAs, 16 MFMAs per iteration.  Output: nanoseconds per MFMA (+ VF FMAs).
+template <int G, int VF>
+__global__ void __launch_bounds__(256, 4) grouped_kernel(float* out, int reps) {
+  constexpr int TOTAL = 16;
+  const int lane = threadIdx.x;
+  bf16x8 a, b;
+  for (int j = 0; j < 8; ++j) { a[j] = (__bf16)(0.01f * (lane + j)); b[j] = (__bf16)(0.02f * (lane - j)); }
+  f32x16 acc[4];
+  for (int i = 0; i < 4; ++i) for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+  float f[32];
+  for (int j = 0; j < 32; ++j) f[j] = 0.001f * (lane + j);
+#pragma unroll 1
+  for (int r = 0; r < reps; ++r) {
+#pragma unroll
+    for (int g = 0; g < TOTAL / G; ++g) {
+#pragma unroll
+      for (int m = 0; m < G; ++m)
+        acc[(g * G + m) & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[(g * G + m) & 3], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int v = 0; v < G * VF; ++v) f[(v + g) & 31] = __builtin_fmaf(f[(v + g) & 31], 0.999f, 0.001f);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  float sum = 0;
+  for (int i = 0; i < 4; ++i) for (int j = 0; j < 16; ++j) sum += acc[i][j];
+  for (int j = 0; j < 32; ++j) sum += f[j];
+  out[blockIdx.x * 256 + threadIdx.x] = sum;
+}
+
+template <int G, int VF>
+static void run_grouped(float* out, int waves_per_simd) {
+  const int reps = 20000;
+  hipEvent_t e0, e1;
+  hipEventCreate(&e0);
+  hipEventCreate(&e1);
+  int cus = 0;
+  hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, 0);
+  hipLaunchKernelGGL((grouped_kernel<G, VF>), dim3(cus * waves_per_simd), dim3(256), 0, 0, out, 10);
+  hipDeviceSynchronize();
+  hipEventRecord(e0);
+  hipLaunchKernelGGL((grouped_kernel<G, VF>), dim3(cus * waves_per_simd), dim3(256), 0, 0, out, reps);
+  hipEventRecord(e1);
+  hipEventSynchronize(e1);
+  float ms = 0.f;
+  hipEventElapsedTime(&ms, e0, e1);
+  std::printf("%d wave(s)/SIMD  %2d MFMA then %3d FMA               %6.2f ns per MFMA + %d FMA\n", waves_per_simd, G, G * VF,
+              ms * 1e6 / reps / waves_per_simd / 16, VF);
+  std::fflush(stdout);
+}
+
 template <int M, int VF, int VT>
 static void run(float* out, int waves_per_simd, const char* what) {
   const int reps = 20000, groups = 16;
@@ -82,6 +134,13 @@ int main() {
     run<1, 0, 2>(out, w, "1 MFMA + 2 EXP2");
     run<1, 0, 4>(out, w, "1 MFMA + 4 EXP2");
     run<1, 4, 2>(out, w, "1 MFMA + 4 FMA + 2 EXP2");
+  }
+  for (int w = 1; w <= 3; ++w) {
+    run_grouped<1, 8>(out, w);
+    run_grouped<4, 8>(out, w);
+    run_grouped<16, 8>(out, w);
+    run_grouped<1, 12>(out, w);
+    run_grouped<16, 12>(out, w);
   }
   hipFree(out);
   return 0;
