@@ -113,18 +113,35 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
 
   // D. emit tiles: slot -> ranked document by binary search over the prefix
   const bool ok = s_status == 0;
+  // The hardware deals workgroups to the CUs round-robin in launch order (workgroups i and
+  // i + number of CUs start on the same CU and run side by side), and hands out the rest as
+  // slots free up.  Equal-length documents are therefore listed tile-major, the most expensive
+  // tile of every document first: all expensive tiles start at once and the cheap ones fill
+  // in behind them.  (Document-major order would put the same tile of every batch entry on
+  // the same CU.)  Packed documents of different lengths stay document-major, which keeps the
+  // K/V rows a workgroup's neighbours read in the caches.
   for (int s = tid; s < total_q && ok; s += SCHED_THREADS) {
-    int lo = 0, hi = nd;   // largest i with qoff[i] <= s
-    while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (qoff[mid] <= s) lo = mid; else hi = mid; }
-    const int d = order[lo];
+    int d, within;   // document, position among its tiles in cost order
+    if (fixed) {
+      d = s % nd;
+      within = s / nd;
+    } else {
+      int lo = 0, hi = nd;   // largest i with qoff[i] <= s
+      while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (qoff[mid] <= s) lo = mid; else hi = mid; }
+      d = order[lo];
+      within = s - qoff[lo];
+    }
     const int nq = cdiv(dlen[d], BM);
     Tile t;
     t.tok_start = fixed ? 0 : dstart[d];
     t.doc_len = dlen[d];
-    t.idx = nq - 1 - (s - qoff[lo]);     // newest (most expensive) query tile first
+    t.idx = nq - 1 - within;             // newest (most expensive) query tile first
     t.batch = fixed ? d : 0;
     qtiles[s] = t;
   }
+  // Key tiles stay document-major for every input: one workgroup per CU runs at a time, so the
+  // hardware hands them out one by one as CUs free up, and neighbours that share a document
+  // share its Q and dO rows in the caches.
   for (int s = tid; s < total_kv && ok; s += SCHED_THREADS) {
     int lo = 0, hi = nd;
     while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (kvoff[mid] <= s) lo = mid; else hi = mid; }
