@@ -5,6 +5,7 @@ argument order, defaults and return values (``sb_attn_varlen`` :71-78, ``sb_attn
 :81-82, ``StickBreakingAttention`` :24-68).  The device work is done by libsba.so.
 """
 import math
+import weakref
 
 import torch
 
@@ -29,6 +30,27 @@ def varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current=Fal
 
 def varlen_bwd(do, dr, q, k, v, state, logit_scale, attend_current=False, fused=False):
     return _ops.run_backward(q, k, v, do, dr, False, state, logit_scale, attend_current, fused=fused)
+
+
+# The last cu_seqlens tensor whose first entry was read back and found to be zero.
+_zero_start_checked = None
+
+
+def _starts_at_zero(cu_seqlens) -> bool:
+    """``cu_seqlens[0] == 0``, upstream's check (sb_varlen/__init__.py:73).  Reading one element of a
+    device tensor stalls the host until the GPU has drained, and a model passes the same
+    cu_seqlens to every layer, so the answer is remembered for as long as the same tensor object
+    comes back unmodified: one synchronisation per batch instead of one per call."""
+    global _zero_start_checked
+    if torch.compiler.is_compiling():
+        return bool(cu_seqlens[0] == 0)
+    seen = _zero_start_checked
+    if seen is not None and seen[0]() is cu_seqlens and seen[1] == cu_seqlens._version:
+        return True
+    ok = bool(cu_seqlens[0] == 0)
+    if ok:
+        _zero_start_checked = (weakref.ref(cu_seqlens), cu_seqlens._version)
+    return ok
 
 
 class StickBreakingAttention(torch.autograd.Function):
@@ -59,7 +81,7 @@ def sb_attn_varlen(q, k, v, cu_seqlens, max_seqlens=None, inv_temp=None, zero_st
     leading 0 when ``zero_start``).  Returns (o [heads, total_tokens, head_dim],
     rem [heads, total_tokens])."""
     if zero_start:
-        assert cu_seqlens[0] == 0
+        assert _starts_at_zero(cu_seqlens)
         cu_seqlens = cu_seqlens[1:]
     if inv_temp is None:
         inv_temp = 1 / math.sqrt(q.size(-1))
@@ -100,7 +122,7 @@ def sb_attn_varlen_fused(q, k, v, cu_seqlens, max_seqlens=None, inv_temp=None, z
     from its two outputs, ``o + rem[..., None] * v`` (upstream tests/test_varlen.py:101), without
     the extra passes over ``o`` and ``v`` in forward and backward."""
     if zero_start:
-        assert cu_seqlens[0] == 0
+        assert _starts_at_zero(cu_seqlens)
         cu_seqlens = cu_seqlens[1:]
     if inv_temp is None:
         inv_temp = 1 / math.sqrt(q.size(-1))

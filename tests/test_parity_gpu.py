@@ -418,3 +418,21 @@ def test_torch_compile_traces_through_the_registered_operators():
     torch.cuda.synchronize()
     for a, b in zip(*outs):
         assert torch.equal(a, b)
+
+
+def test_zero_start_check_is_remembered_per_tensor():
+    """The leading-zero assertion reads the device once per cu_seqlens tensor, not once per call, and
+    still fires for a new or modified tensor."""
+    from stickbreaking_attention import sb_attn_varlen
+    from stickbreaking_attention import sb_varlen
+    q = torch.zeros(2, 256, 64, dtype=torch.bfloat16, device=DEV)
+    cu = torch.tensor([0, 100, 256], dtype=torch.int32, device=DEV)
+    sb_attn_varlen(q, q, q, cu, 256)
+    assert sb_varlen._zero_start_checked[0]() is cu
+    sb_attn_varlen(q, q, q, cu, 256)                       # same tensor: no second read
+    cu[0] = 3                                              # in-place change bumps the version: checked again
+    with pytest.raises(AssertionError):
+        sb_attn_varlen(q, q, q, cu, 256)
+    with pytest.raises(AssertionError):
+        sb_attn_varlen(q, q, q, torch.tensor([5, 256], dtype=torch.int32, device=DEV), 256)
+    torch.cuda.synchronize()
