@@ -122,3 +122,18 @@ def test_operators_are_registered_under_the_upstream_names():
     import stickbreaking_attention  # noqa: F401
     for name in ("varlen_fwd", "varlen_bwd", "attn_fwd", "attn_bwd"):
         assert hasattr(torch.ops.stickbreaking_attention, name)
+
+
+def test_leading_zero_check_is_cached_per_tensor_object():
+    """Host logic only: the answer for one cu_seqlens tensor is reused until the tensor is modified
+    in place or another tensor arrives (upstream asserts on every call, sb_varlen/__init__.py:73)."""
+    import torch
+    from stickbreaking_attention import sb_varlen
+    cu = torch.tensor([0, 5, 9], dtype=torch.int32)
+    assert sb_varlen._starts_at_zero(cu)
+    assert sb_varlen._zero_start_checked[0]() is cu
+    same_values = torch.tensor([0, 5, 9], dtype=torch.int32)
+    assert sb_varlen._starts_at_zero(same_values) and sb_varlen._zero_start_checked[0]() is same_values
+    same_values[0] = 2
+    assert not sb_varlen._starts_at_zero(same_values)
+    assert not sb_varlen._starts_at_zero(torch.tensor([1, 4]))
