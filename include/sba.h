@@ -151,6 +151,22 @@ int sba_attn_fwd_weights(const sba_problem* p, const void* schedule,
                          const sba_view* o, const sba_view* rem,
                          float* stick_table, float* weights, void* stream);
 
+/* Forward of packed variable-length input for callers that cannot allocate device memory (code
+ * running under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart upstream, where PyTorch allocates every buffer.  Same results as
+ * sba_build_schedule + sba_varlen_fwd with stick_table == NULL (no backward can follow), but the
+ * schedule workspace is a fixed array of SBA_STATIC_SCRATCH_BYTES bytes that lives inside the
+ * library's code object on every GPU it runs on, from the first call until the process ends; the
+ * call allocates and frees nothing.  Problems whose sba_schedule_bytes() exceed that size are
+ * rejected with SBA_E_WORKSPACE (the array holds, for example, 262144 tokens in 8192 documents).
+ * All calls on one GPU share that GPU's array: calls that overlap on one GPU (different streams
+ * or threads) race; serialise them.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress): make that call outside any graph capture. */
+#define SBA_STATIC_SCRATCH_BYTES (512 * 1024)
+int sba_varlen_fwd_static(const sba_problem* p,
+                          const sba_view* q, const sba_view* k, const sba_view* v,
+                          const sba_view* o, const sba_view* rem, void* stream);
+
 /* ---- backward --------------------------------------------------------------------------- */
 
 /* dq, dk, dv for every token (zero for tokens that belong to no document).  `stick_table` is the

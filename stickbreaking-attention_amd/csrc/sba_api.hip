@@ -91,7 +91,7 @@ struct Timer {
   hipStream_t s;
   int which;
   bool on;
-  Timer(int which_, hipStream_t s_) : s(s_), which(which_), on(g_timing.load() != 0) {
+  Timer(int which_, hipStream_t s_, bool allowed = true) : s(s_), which(which_), on(allowed && g_timing.load() != 0) {
     if (on) {
       on = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess;
       if (on) (void)hipEventRecord(e0, s);
@@ -126,7 +126,8 @@ int fill_common(const sba_problem* p, const Sizes& sz, const void* schedule, KAr
 }
 
 int forward(const sba_problem* p, bool fixed, const void* schedule, const sba_view* q, const sba_view* k,
-            const sba_view* v, const sba_view* o, const sba_view* rem, float* stick, float* weights, void* stream) {
+            const sba_view* v, const sba_view* o, const sba_view* rem, float* stick, float* weights, void* stream,
+            bool timed = true) {
   Sizes sz;
   int e = check_problem(p, fixed, &sz);
   if (e) return e;
@@ -143,7 +144,7 @@ int forward(const sba_problem* p, bool fixed, const void* schedule, const sba_vi
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   hipError_t he = hipSuccess;
   if (sz.n_docs > 0) {
-    Timer tm(0, s);
+    Timer tm(0, s, timed);
     he = launch_fwd(a, p->head_dim, (p->flags & SBA_ATTEND_CURRENT) != 0,
                     (p->flags & SBA_PRODUCT_SPACE) != 0, weights != nullptr, sz.n_q_max, s);
   }
@@ -195,6 +196,31 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, const sba_v
   z.mat[0] = a.dq; z.mat[1] = a.dk; z.mat[2] = a.dv; z.n_mat = 3;
   z.sched = a.sched; z.heads = p->heads; z.tokens = p->tokens; z.head_dim = p->head_dim;
   return (int)launch_zero_tail(z, s);
+}
+
+// Schedule workspace of sba_varlen_fwd_static: one array per GPU, inside the code object, so the
+// entry point needs no allocation.  In host code the name `scratch` is only a handle for
+// hipGetSymbolAddress; kernels get the device address looked up once per device.
+static __device__ __align__(256) unsigned char scratch[SBA_STATIC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::atomic<void*> g_scratch_ptr[MAX_DEVICES];
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t he = hipGetDevice(&dev);
+  if (he != hipSuccess) return (int)he;
+  if (dev < 0 || dev >= MAX_DEVICES) return SBA_E_ARCH;
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    he = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (he != hipSuccess) return (int)he;
+    if (ptr == nullptr) return SBA_E_NULL;
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);   // every thread computes the same address
+  }
+  *out = ptr;
+  return 0;
 }
 
 }  // namespace
@@ -288,6 +314,21 @@ int sba_attn_bwd(const sba_problem* p, const void* schedule, const sba_view* q, 
                  const float* stick_table, float* grad_table, const sba_view* dq, const sba_view* dk,
                  const sba_view* dv, void* stream) {
   return backward(p, true, schedule, q, k, v, grad_o, grad_rem, stick_table, grad_table, dq, dk, dv, stream);
+}
+
+int sba_varlen_fwd_static(const sba_problem* p, const sba_view* q, const sba_view* k, const sba_view* v,
+                          const sba_view* o, const sba_view* rem, void* stream) {
+  Sizes sz;
+  int e = check_problem(p, false, &sz);
+  if (e) return e;
+  if (schedule_bytes(sz) > (size_t)SBA_STATIC_SCRATCH_BYTES) return SBA_E_WORKSPACE;
+  if ((e = check_arch())) return e;
+  void* sched = nullptr;
+  if ((e = static_scratch(&sched))) return e;
+  // The scheduler rewrites the header and every list entry the kernels will use; nothing of
+  // the previous call's contents is read, so nothing needs clearing.
+  if ((e = sba_build_schedule(p, sched, stream))) return e;
+  return forward(p, false, sched, q, k, v, o, rem, nullptr, nullptr, stream, /*timed=*/false);   // (timing creates events)
 }
 
 void sba_set_timing(int on) { g_timing.store(on); }

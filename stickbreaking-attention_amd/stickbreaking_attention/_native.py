@@ -45,7 +45,7 @@ class SbaProblem(ctypes.Structure):
 EXPORTS = (
     "sba_version", "sba_error_string", "sba_schedule_bytes", "sba_table_bytes", "sba_build_schedule",
     "sba_varlen_fwd", "sba_varlen_bwd", "sba_attn_fwd", "sba_attn_bwd", "sba_set_timing",
-    "sba_last_kernel_ms", "sba_varlen_fwd_weights", "sba_attn_fwd_weights",
+    "sba_last_kernel_ms", "sba_varlen_fwd_weights", "sba_attn_fwd_weights", "sba_varlen_fwd_static",
 )
 
 _lib = None
@@ -87,6 +87,8 @@ def load():
             f = getattr(lib, name)
             f.restype = ctypes.c_int
             f.argtypes = [P, vp, V, V, V, V, V, vp, vp, V, V, V, vp]
+        lib.sba_varlen_fwd_static.restype = ctypes.c_int
+        lib.sba_varlen_fwd_static.argtypes = [P, V, V, V, V, V, vp]
         lib.sba_set_timing.restype = None
         lib.sba_set_timing.argtypes = [ctypes.c_int]
         lib.sba_last_kernel_ms.restype = ctypes.c_float
