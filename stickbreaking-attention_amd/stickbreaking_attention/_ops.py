@@ -16,6 +16,7 @@ buffers the caller allocated, so they need no shape function.
 import ctypes
 import math
 import os
+import warnings
 from typing import Optional, Tuple
 
 import torch
@@ -57,11 +58,26 @@ def workspace_sizes(fixed: bool, batch: int, heads: int, tokens: int, n_docs: in
     return (4 * words + 255) & ~255, heads * (n_tt + 1) * rows
 
 
+_warned_dtypes = set()
+
+
+def _warn_reduced_precision(dtype) -> None:
+    """Upstream runs its dots in the input dtype (tl.dot on fp16 / TF32 on fp32 inputs,
+    sb_varlen_fwd.py:42, utils.py:8); this library multiplies in bf16 whatever arrives.  Said once
+    per dtype instead of silently."""
+    if dtype not in _warned_dtypes:
+        _warned_dtypes.add(dtype)
+        warnings.warn(f"stickbreaking_attention: {dtype} inputs are rounded to bfloat16 before the matrix products "
+                      "(8 bits of mantissa; outputs are returned in the input dtype)", stacklevel=4)
+
+
 def _prep(t: torch.Tensor, dpad: int, incoming_grad: bool = False) -> torch.Tensor:
     """bf16, head_dim padded with zeros to `dpad`, row strides multiples of 8 elements (traceable).
     The strides of an incoming gradient are not known while a backward is being traced, so
     there it is simply made contiguous."""
     if t.dtype != torch.bfloat16:
+        if not torch.compiler.is_compiling():
+            _warn_reduced_precision(t.dtype)
         t = t.to(torch.bfloat16)
     d = t.shape[-1]
     if d != dpad:

@@ -36,20 +36,35 @@ def varlen_bwd(do, dr, q, k, v, state, logit_scale, attend_current=False, fused=
 _zero_start_checked = None
 
 
+def _version_of(t):
+    """The in-place modification counter of a tensor, or None where PyTorch keeps none (tensors
+    created under ``torch.inference_mode()`` raise on ``_version``)."""
+    try:
+        return t._version
+    except RuntimeError:
+        return None
+
+
 def _starts_at_zero(cu_seqlens) -> bool:
     """``cu_seqlens[0] == 0``, upstream's check (sb_varlen/__init__.py:73).  Reading one element of a
     device tensor stalls the host until the GPU has drained, and a model passes the same
     cu_seqlens to every layer, so the answer is remembered for as long as the same tensor object
-    comes back unmodified: one synchronisation per batch instead of one per call."""
+    comes back unmodified: one synchronisation per batch instead of one per call.  Tensors without
+    a modification counter (inference tensors) are checked on every call.  A write through
+    ``cu_seqlens.data`` does not advance the counter and is therefore not seen: do not rewrite a
+    cu_seqlens tensor that way between calls."""
     global _zero_start_checked
     if torch.compiler.is_compiling():
         return bool(cu_seqlens[0] == 0)
+    version = _version_of(cu_seqlens)
+    if version is None:
+        return bool(cu_seqlens[0] == 0)
     seen = _zero_start_checked
-    if seen is not None and seen[0]() is cu_seqlens and seen[1] == cu_seqlens._version:
+    if seen is not None and seen[0]() is cu_seqlens and seen[1] == version:
         return True
     ok = bool(cu_seqlens[0] == 0)
     if ok:
-        _zero_start_checked = (weakref.ref(cu_seqlens), cu_seqlens._version)
+        _zero_start_checked = (weakref.ref(cu_seqlens), version)
     return ok
 
 

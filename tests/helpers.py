@@ -31,17 +31,51 @@ def err_stats(name, got, ref):
     return {"name": name, "max_abs": diff.max().item() if diff.numel() else 0.0, "median_rel": rel}
 
 
-def assert_close(name, got, ref, tol=TOL):
-    """max-abs gate.  The kernels return bf16, whose own rounding is up to |x| * 2^-8 (0.031
-    for |x| in [8, 16)), so on top of the absolute tolerance an element may differ by half a
-    bf16 ulp of the reference value; for |ref| < 2.5 the bound is the plain 2e-2 to within 1e-2."""
+def assert_close(name, got, ref, tol=TOL, scale=1.0):
+    """The parity gate.  Flat part: max-abs error <= 2e-2 -- asserted as is for ``rem`` and for every
+    tensor whose reference values stay below 2.5 in magnitude.  Larger values cannot meet a flat
+    bound in bf16 at all (the rounding of the OUTPUT alone is up to |x| * 2^-8: 1.6e-2 at |x| = 4,
+    3.1e-2 at 8), so there an element may additionally differ by half a bf16 ulp of the
+    reference value.  ``scale`` > 1 widens the flat part for inputs hotter than N(0,1): the error
+    of rounding the bf16 MFMA operands P and dZ grows with the cube of the input scale (dz ~
+    scale^2, k ~ scale; oracle/rounding_model.py reproduces it on the CPU).  Prints, per tensor,
+    the max-abs error, the median relative error, and how many elements exceed the flat 2e-2."""
     assert torch.isfinite(got.float()).all(), f"{name}: non-finite values"
     s = err_stats(name, got, ref)
     g, r = got.detach().float().cpu(), ref.detach().float().cpu()
-    excess = ((g - r).abs() - (tol + r.abs() * 2.0 ** -8)).max().item() if g.numel() else -1.0
-    print(f"  {name}: max_abs={s['max_abs']:.3e} median_rel={s['median_rel']:.3e} max|ref|={r.abs().max().item() if r.numel() else 0:.2f}")
-    assert excess <= 0, f"{name}: error exceeds {tol} + bf16 half-ulp by {excess:.4e} (max_abs {s['max_abs']:.4e})"
+    flat = tol * max(1.0, float(scale)) ** 3
+    diff = (g - r).abs()
+    max_ref = r.abs().max().item() if r.numel() else 0.0
+    over_flat = int((diff > TOL).sum()) if g.numel() else 0
+    excess_flat = (diff - flat).max().item() if g.numel() else -1.0
+    excess = (diff - (flat + r.abs() * 2.0 ** -8)).max().item() if g.numel() else -1.0
+    s.update(max_ref=max_ref, over_flat=over_flat, numel=g.numel())
+    print(f"  {name}: max_abs={s['max_abs']:.3e} median_rel={s['median_rel']:.3e} max|ref|={max_ref:.2f} "
+          f"over_flat_2e-2={over_flat}/{g.numel()}")
+    if name == "rem" or max_ref < 2.5:
+        assert excess_flat <= 0, f"{name}: error exceeds the flat {flat:g} by {excess_flat:.4e} (max_abs {s['max_abs']:.4e})"
+    assert excess <= 0, f"{name}: error exceeds {flat:g} + bf16 half-ulp by {excess:.4e} (max_abs {s['max_abs']:.4e})"
     return s
+
+
+def assert_matches_rounding_model(names, got, q, k, v, do, lengths, drem=None, attend_current=False, inv_temp=None):
+    """Compare with oracle/rounding_model.py (float64 arithmetic with the kernels' bf16 rounding
+    points).  What may still differ: fp32 against float64 accumulation, which now and then moves an
+    operand or an output across a bf16 rounding boundary -- one bf16 ulp of the value (2^-7 relative)
+    plus a small absolute term."""
+    from oracle import rounding_model as rm
+    model = dict(zip(("o", "rem", "dq", "dk", "dv"),
+                     rm.varlen(q.cpu(), k.cpu(), v.cpu(), do.cpu(), lengths, None if drem is None else drem.cpu(),
+                               attend_current, inv_temp)))
+    worst = {}
+    for name, g in zip(names, got):
+        m = model[name]
+        diff = (g.detach().double().cpu() - m).abs()
+        bound = 6e-3 + m.abs() * 2.0 ** -7
+        worst[name] = diff.max().item()
+        print(f"  {name} vs rounding model: max_abs={worst[name]:.3e}")
+        assert (diff <= bound).all(), f"{name}: differs from the rounding model by {(diff - bound).max().item():.3e} beyond one bf16 ulp"
+    return worst
 
 
 def oracle_varlen(q, k, v, do, lengths, attend_current=False, inv_temp=None, drem=None, row_chunk=0):

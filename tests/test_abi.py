@@ -137,3 +137,17 @@ def test_leading_zero_check_is_cached_per_tensor_object():
     same_values[0] = 2
     assert not sb_varlen._starts_at_zero(same_values)
     assert not sb_varlen._starts_at_zero(torch.tensor([1, 4]))
+
+
+def test_leading_zero_check_works_on_inference_tensors():
+    """Tensors created under torch.inference_mode() have no version counter: the check must fall
+    back to reading the first element every time instead of raising."""
+    import torch
+    from stickbreaking_attention import sb_varlen
+    with torch.inference_mode():
+        cu = torch.tensor([0, 5, 9], dtype=torch.int32)
+        bad = torch.tensor([3, 5, 9], dtype=torch.int32)
+        assert sb_varlen._starts_at_zero(cu) and sb_varlen._starts_at_zero(cu)
+        assert not sb_varlen._starts_at_zero(bad)
+    assert sb_varlen._starts_at_zero(cu)          # also outside the mode, on the inference tensor
+    assert sb_varlen._zero_start_checked is None or sb_varlen._zero_start_checked[0]() is not cu

@@ -1,0 +1,92 @@
+"""The edges of the supported input envelope: logits far outside N(0,1) in both carry spaces,
+genuinely fp32 inputs, and upstream's own long single-document case (tests/test_varlen.py:68-93:
+one 16384-token document, head_dim 128, shifted q/k that keep weight alive hundreds of keys
+from the diagonal)."""
+import os
+import warnings
+
+import pytest
+import torch
+
+from oracle import sb_oracle as orc
+from tests.helpers import assert_close, assert_matches_rounding_model, cu_from_lengths, oracle_varlen
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from stickbreaking_attention import _native as nat
+    assert os.path.exists(nat.LIB_PATH), "libsba.so must be built before the GPU tests run"
+    nat.load()
+
+
+def _run(q, k, v, do, lengths, ac=False):
+    from stickbreaking_attention import sb_attn_varlen
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    cu = cu_from_lengths(lengths, device=DEV)
+    o, rem = sb_attn_varlen(qg, kg, vg, cu, max(lengths), zero_start=False, attend_current=ac)
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do.to(DEV))
+    torch.cuda.synchronize()
+    return o.detach(), rem.detach(), dq, dk, dv
+
+
+@pytest.mark.parametrize("product_space", [False, True])
+@pytest.mark.parametrize("qk_scale", [3.0, 8.0])
+@pytest.mark.parametrize("d", [64, 128])
+def test_large_logits(product_space, qk_scale, d, monkeypatch):
+    """q and k scaled so that the logits reach +-35 (x3) or +-250 (x8): sigmoid saturates, 2^z
+    overflows fp32 (product space: r = 0; log2 space: logit clamped at 126), the forward's clamp
+    of the odds at 2^30 and the backward's unclamped 1 - sigmoid differ by at most 2^-30.
+    Everything must stay finite and agree with the oracle; the gate is widened as for any
+    hot input (dq and dk carry the factor of k resp. q)."""
+    from stickbreaking_attention import _ops
+    monkeypatch.setattr(_ops, "PRODUCT_SPACE", product_space)
+    lengths = [300, 129, 64]
+    q, k, v, do = orc.make_inputs((2, sum(lengths), d), 500 + d)
+    q, k = (q.float() * qk_scale).to(torch.bfloat16), (k.float() * qk_scale).to(torch.bfloat16)
+    for ac in (False, True):
+        got = _run(q, k, v, do, lengths, ac)
+        ref = oracle_varlen(q, k, v, do, lengths, ac)
+        for name, g, r in zip(("o", "rem", "dq", "dk", "dv"), got, ref):
+            assert_close(name, g, r, scale=qk_scale ** (1.0 / 3.0) if name in ("dq", "dk") else 1.0)
+        assert_matches_rounding_model(("o", "rem", "dq", "dk", "dv"), got, q, k, v, do, lengths, None, ac)
+
+
+def test_fp32_inputs_are_rounded_to_bf16_and_say_so():
+    """fp32 N(0,1) inputs that are NOT bf16-representable, against the oracle on those fp32
+    values: the library rounds q, k, v, grad_o to bf16 (and warns once per dtype).  Rounding the
+    inputs moves every logit by about 2^-9 sqrt(2) |z|, which stays inside the usual gate."""
+    from stickbreaking_attention import _ops, sb_attn_varlen
+    _ops._warned_dtypes.discard(torch.float32)
+    lengths = [257, 640, 95]
+    T = sum(lengths)
+    g = torch.Generator().manual_seed(4321)
+    q, k, v, do = (torch.randn((3, T, 64), generator=g) for _ in range(4))
+    assert not torch.equal(q, q.to(torch.bfloat16).float())
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    cu = cu_from_lengths(lengths, device=DEV)
+    with pytest.warns(UserWarning, match="rounded to bfloat16"):
+        o, rem = sb_attn_varlen(qg, kg, vg, cu, max(lengths), zero_start=False)
+    assert o.dtype == torch.float32 and rem.dtype == torch.float32
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")          # said once, not on every call
+        dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do.to(DEV))
+    torch.cuda.synchronize()
+    ref = orc.sb_varlen_grads(q, k, v, lengths, do)
+    for name, gt, r in zip(("o", "rem", "dq", "dk", "dv"), (o.detach(), rem.detach(), dq, dk, dv), ref):
+        assert_close(name + " (fp32 inputs)", gt, r)
+
+
+def test_upstream_single_16k_document():
+    """One 16384-token document, head_dim 128, upstream's shifted distribution, forward and
+    backward; the oracle checks both heads, 1024 query rows at a time."""
+    L = 16384
+    q, k, v, do = orc.make_inputs((2, L, 128), 1337, dist="upstream")
+    got = _run(q, k, v, do, [L])
+    ref = oracle_varlen(q, k, v, do, [L], row_chunk=1024)
+    for name, g, r in zip(("o", "rem", "dq", "dk", "dv"), got, ref):
+        assert_close(name, g, r)

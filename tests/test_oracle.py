@@ -197,3 +197,24 @@ def test_package_dense_definition_matches_the_oracle():
         o1, r1 = dense(q, k, v, mask, cw)
         o2, r2 = orc.stickbreaking(q, k, v, mask, cw)
         assert torch.allclose(o1, o2, atol=1e-10) and torch.allclose(r1, r2, atol=1e-10)
+
+
+def test_varlen_grads_match_bruteforce_and_analytic_backward_per_document():
+    # the check the golden-fixture generator relies on: autograd through the packed-documents
+    # driver == product-form double loop (forward) and hand-derived formulas (backward), per document
+    H, lengths, d = 2, [70, 1, 150, 33], 16
+    T = sum(lengths)
+    for ac in (False, True):
+        q, k, v, do = (t.double() for t in orc.make_inputs((H, T, d), 4242 + T, dist="upstream"))
+        dr = torch.randn((H, T), generator=torch.Generator().manual_seed(99 + T)).to(torch.bfloat16).double()
+        o, rem, dq, dk, dv = orc.sb_varlen_grads(q, k, v, lengths, do, dr, ac)
+        start = 0
+        for n in lengths:
+            sl = slice(start, start + n)
+            for h in range(H):
+                ob, rb, _ = orc.bruteforce(q[h, sl], k[h, sl], v[h, sl], ac)
+                assert torch.allclose(o[h, sl], ob, atol=1e-11) and torch.allclose(rem[h, sl], rb, atol=1e-11)
+                aq, ak, av = orc.analytic_backward(q[h, sl], k[h, sl], v[h, sl], do[h, sl], dr[h, sl], ac)
+                assert torch.allclose(dq[h, sl], aq, atol=1e-10) and torch.allclose(dk[h, sl], ak, atol=1e-10)
+                assert torch.allclose(dv[h, sl], av, atol=1e-10)
+            start += n
