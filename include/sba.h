@@ -24,7 +24,10 @@
  * that ownership model.  What differs is the private state carried from forward to
  * backward: instead of one fp32 log-remainder per row (upstream `neg_log_acc`) the forward
  * fills a per-(row, 32-key block) carry table that both backward kernels consume, so the
- * backward needs neither locks nor atomics.
+ * backward needs neither locks nor atomics.  Every workspace is passed with its size in bytes;
+ * an entry point never reads or writes past a size it was given: what the host can check comes
+ * back as SBA_E_WORKSPACE, what only the device can know (the documents inside cu_seqlens) makes
+ * the kernels return early and the outputs NaN.
  */
 #ifndef SBA_H_
 #define SBA_H_
@@ -36,7 +39,7 @@
 extern "C" {
 #endif
 
-#define SBA_VERSION 101
+#define SBA_VERSION 200
 
 /* error codes (negative returns) */
 #define SBA_E_NULL      (-1)  /* a required pointer is NULL                         */
@@ -45,7 +48,10 @@ extern "C" {
 #define SBA_E_SHAPE     (-4)  /* negative / inconsistent sizes, or tokens*stride_t
                                  too large for 32-bit byte offsets (>= 2 GiB)       */
 #define SBA_E_STRIDE    (-5)  /* a row start is not 16-byte aligned (stride % 8)    */
-#define SBA_E_WORKSPACE (-6)  /* workspace or table too small                       */
+#define SBA_E_WORKSPACE (-6)  /* a workspace handed in is smaller than the problem
+                                 needs: schedule, weights array, the tables of the
+                                 fixed-length op, the static array of
+                                 sba_varlen_fwd_static                              */
 #define SBA_E_ARCH      (-7)  /* current device is not gfx950                       */
 
 /* element types */
@@ -77,7 +83,7 @@ typedef struct sba_view {
   int64_t stride_t;
 } sba_view;
 
-/* Problem description shared by all four entry points. */
+/* Problem description shared by all entry points. */
 typedef struct sba_problem {
   int32_t  dtype;        /* SBA_BF16                                                     */
   int32_t  head_dim;     /* 64 or 128                                                    */
@@ -85,9 +91,10 @@ typedef struct sba_problem {
   int32_t  batch;        /* B for the fixed-length op, 1 for varlen                      */
   int32_t  tokens;       /* T: tokens per batch entry (fixed) / total packed tokens      */
   int32_t  n_docs;       /* varlen: number of entries in cu_seqlens; fixed: ignored      */
-  int32_t  max_doc_len;  /* upper bound on any document length (fixed: == tokens); sizes
-                            the carry tables: a longer document makes the scheduler flag
-                            SBA_STATUS_DOC_TOO_LONG and all kernels return early         */
+  int32_t  max_doc_len;  /* upper bound on any document length (fixed: == tokens; 0 =
+                            unknown).  Only sba_table_bytes() looks at it; results never
+                            depend on it (upstream drops rows when its max_seqlens is
+                            too small, sb_varlen_fwd.py:478)                             */
   uint32_t flags;        /* SBA_ATTEND_CURRENT | SBA_CU_INT64 | SBA_PRODUCT_SPACE | ...  */
   float    inv_temp;     /* logit scale (upstream logit_scale / inv_temp)                */
   const void* cu_seqlens;/* varlen: inclusive cumulative document ends, WITHOUT a leading
@@ -99,57 +106,73 @@ typedef struct sba_problem {
 /* Bytes of the schedule workspace (tile lists + status words) for this problem. */
 size_t sba_schedule_bytes(const sba_problem* p);
 
-/* Bytes of ONE carry table (fp32 [heads][ceil(max_doc_len/32) + 1][batch*tokens]; the last
- * plane holds one value per row: rem, resp. the complete gradient of rem).  The forward
- * fills `stick_table`; the backward additionally needs a `grad_table` of the same size. */
+/* Bytes of ONE carry table.  A table holds, per head and per document of length L, one fp32 for
+ * every (32-key block, query row at or below it) pair -- about L*L/64 -- plus one per row (the
+ * forward leaves rem there in fp32, the backward the complete gradient of rem).  The forward
+ * fills `stick_table`; the backward additionally needs a `grad_table` of the same size.
+ *   sba_table_bytes              no lengths needed: the most any documents of at most
+ *                                max_doc_len tokens can need (exact for the fixed-length op);
+ *   sba_table_bytes_for_lengths  exact, from the document lengths in HOST memory.
+ * Tables may be larger than needed.  Tables that turn out too small for the documents in
+ * cu_seqlens (a max_doc_len that under-states them) are detected on the device: nothing runs
+ * and every output is filled with NaN (see SBA_STATUS_TABLE_TOO_SMALL). */
 size_t sba_table_bytes(const sba_problem* p);
+size_t sba_table_bytes_for_lengths(const sba_problem* p, const int64_t* doc_lengths, int n_lengths);
 
 /* ---- schedule --------------------------------------------------------------------------- */
 
 /* Builds, on the device, the list of 128-row query tiles and 128-key KV tiles from
- * cu_seqlens (documents sorted longest first, tiles of a document newest first) and validates
- * cu_seqlens.  `schedule` must hold sba_schedule_bytes() bytes and be 16-byte aligned.  The first int32 of the
- * workspace is a status word (0 = ok, else SBA_STATUS_*), readable by the caller after the
- * stream has drained.  Has no upstream counterpart as a separate call: upstream derives the
- * tile of a program from its grid index inside `_forward` (sb_varlen_fwd.py:281-296). */
-int sba_build_schedule(const sba_problem* p, void* schedule, void* stream);
+ * cu_seqlens (documents sorted longest first, tiles of a document newest first), assigns every
+ * document its area of the carry tables and validates cu_seqlens.  `schedule` must be 16-byte
+ * aligned and `schedule_size` (its size in bytes) at least sba_schedule_bytes(), else
+ * SBA_E_WORKSPACE.  The first int32 of the workspace is a status word (0 = ok, else
+ * SBA_STATUS_*) and the fourth the number of table entries per head the documents need, both
+ * readable by the caller after the stream has drained.  Has no upstream counterpart as a
+ * separate call: upstream derives the tile of a program from its grid index inside `_forward`
+ * (sb_varlen_fwd.py:281-296). */
+int sba_build_schedule(const sba_problem* p, void* schedule, size_t schedule_size, void* stream);
 
-#define SBA_STATUS_OK            0
-#define SBA_STATUS_BAD_CU        1   /* cu_seqlens not monotone or beyond `tokens`          */
-#define SBA_STATUS_DOC_TOO_LONG  2   /* a document is longer than max_doc_len               */
+#define SBA_STATUS_OK               0
+#define SBA_STATUS_BAD_CU           1   /* cu_seqlens not monotone or beyond `tokens`        */
+#define SBA_STATUS_TABLE_TOO_SMALL  4   /* reported by the Python layer when the fourth header
+                                           word exceeds the entries per head of the tables   */
 
 /* ---- forward ---------------------------------------------------------------------------- */
 
 /* o[b,h,t,:] and rem[b,h,t] for every token: tokens that belong to no document (past the
- * last entry of cu_seqlens) are set to zero, as is everything when the scheduler rejected
- * cu_seqlens.  `stick_table` may be NULL when no
- * backward will follow. */
-int sba_varlen_fwd(const sba_problem* p, const void* schedule,
+ * last entry of cu_seqlens) are set to zero.  When the scheduler rejected cu_seqlens, or
+ * `stick_table` is too small for the documents, no attention is computed and every element of
+ * both outputs is NaN.  `stick_table` (`table_size` bytes) may be NULL when no backward will
+ * follow.  `schedule_size` is checked against sba_schedule_bytes(). */
+int sba_varlen_fwd(const sba_problem* p, const void* schedule, size_t schedule_size,
                    const sba_view* q, const sba_view* k, const sba_view* v,
                    const sba_view* o, const sba_view* rem,
-                   float* stick_table, void* stream);
+                   float* stick_table, size_t table_size, void* stream);
 
-int sba_attn_fwd(const sba_problem* p, const void* schedule,
+int sba_attn_fwd(const sba_problem* p, const void* schedule, size_t schedule_size,
                  const sba_view* q, const sba_view* k, const sba_view* v,
                  const sba_view* o, const sba_view* rem,
-                 float* stick_table, void* stream);
+                 float* stick_table, size_t table_size, void* stream);
 
 /* Debug variants that additionally write the attention weights A[i,j] (fp32, before the bf16
  * rounding that feeds A.V) of every causal in-document pair into `weights`, a dense
- * [batch][heads][tokens][tokens] array (row = query token, column = key token; packed
- * variable-length input: batch == 1 and both indices are positions in the packed sequence).
- * Elements outside the causal triangle of a document are not written: clear the array first.
- * Replaces upstream's `return_attention=True` launches (sb_varlen_fwd.py:195-202, :421-425;
- * sb_attn/sb_fwd.py:147-151).  Quadratic memory; a separate, slower kernel instantiation. */
-int sba_varlen_fwd_weights(const sba_problem* p, const void* schedule,
+ * [batch][heads][tokens][tokens] array of `weights_size` bytes (row = query token, column = key
+ * token; packed variable-length input: batch == 1 and both indices are positions in the packed
+ * sequence).  Elements outside the causal triangle of a document are not written: clear the
+ * array first.  Replaces upstream's `return_attention=True` launches (sb_varlen_fwd.py:195-202,
+ * :421-425; sb_attn/sb_fwd.py:147-151).  Quadratic memory; a separate, slower kernel
+ * instantiation. */
+int sba_varlen_fwd_weights(const sba_problem* p, const void* schedule, size_t schedule_size,
                            const sba_view* q, const sba_view* k, const sba_view* v,
                            const sba_view* o, const sba_view* rem,
-                           float* stick_table, float* weights, void* stream);
+                           float* stick_table, size_t table_size,
+                           float* weights, size_t weights_size, void* stream);
 
-int sba_attn_fwd_weights(const sba_problem* p, const void* schedule,
+int sba_attn_fwd_weights(const sba_problem* p, const void* schedule, size_t schedule_size,
                          const sba_view* q, const sba_view* k, const sba_view* v,
                          const sba_view* o, const sba_view* rem,
-                         float* stick_table, float* weights, void* stream);
+                         float* stick_table, size_t table_size,
+                         float* weights, size_t weights_size, void* stream);
 
 /* Forward of packed variable-length input for callers that cannot allocate device memory (code
  * running under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
@@ -169,20 +192,21 @@ int sba_varlen_fwd_static(const sba_problem* p,
 
 /* ---- backward --------------------------------------------------------------------------- */
 
-/* dq, dk, dv for every token (zero for tokens that belong to no document).  `stick_table` is the
- * table the forward filled for the same problem and inputs; `grad_table` is scratch of the
- * same size.  grad_rem may have ptr == NULL (treated as zeros). */
-int sba_varlen_bwd(const sba_problem* p, const void* schedule,
+/* dq, dk, dv for every token (zero for tokens that belong to no document; NaN everywhere when
+ * nothing could run, as in the forward).  `schedule` and `stick_table` are the ones the forward
+ * of the same problem and inputs filled; `grad_table` is scratch; `table_size` is the size in
+ * bytes of EACH of the two tables.  grad_rem may have ptr == NULL (treated as zeros). */
+int sba_varlen_bwd(const sba_problem* p, const void* schedule, size_t schedule_size,
                    const sba_view* q, const sba_view* k, const sba_view* v,
                    const sba_view* grad_o, const sba_view* grad_rem,
-                   const float* stick_table, float* grad_table,
+                   const float* stick_table, float* grad_table, size_t table_size,
                    const sba_view* dq, const sba_view* dk, const sba_view* dv,
                    void* stream);
 
-int sba_attn_bwd(const sba_problem* p, const void* schedule,
+int sba_attn_bwd(const sba_problem* p, const void* schedule, size_t schedule_size,
                  const sba_view* q, const sba_view* k, const sba_view* v,
                  const sba_view* grad_o, const sba_view* grad_rem,
-                 const float* stick_table, float* grad_table,
+                 const float* stick_table, float* grad_table, size_t table_size,
                  const sba_view* dq, const sba_view* dk, const sba_view* dv,
                  void* stream);
 
@@ -191,10 +215,13 @@ int sba_attn_bwd(const sba_problem* p, const void* schedule,
 int         sba_version(void);
 const char* sba_error_string(int code);
 
-/* Duration in milliseconds of the most recent launch of each kernel (process-wide: the
- * backward may run on another thread), measured with HIP events on the caller's stream when timing is switched on
- * (sba_set_timing(1)); used by the benchmark to time the dominant kernel where it runs.
- * which: 0 = forward, 1 = backward dq pass, 2 = backward dk/dv pass.  Synchronises. */
+/* Benchmark instrumentation, NOT part of the re-entrant interface: with the switch on, every
+ * compute launch is bracketed by HIP events on the caller's stream and the call WAITS for the
+ * kernel (host synchronisation, event creation); sba_last_kernel_ms returns the duration in
+ * milliseconds of the most recent launch of each kernel (which: 0 = forward, 1 = backward dq pass,
+ * 2 = backward dk/dv pass).  One process-wide switch and one process-wide set of results (the
+ * backward may run on PyTorch's autograd thread): do not use with concurrent callers, under
+ * graph capture, or in production.  Off by default; sba_varlen_fwd_static ignores it. */
 void  sba_set_timing(int on);
 float sba_last_kernel_ms(int which);
 

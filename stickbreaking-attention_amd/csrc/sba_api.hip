@@ -21,7 +21,7 @@ inline int cdiv_i(long long a, long long b) { return (int)((a + b - 1) / b); }
 struct Sizes {
   int n_docs;        // documents the scheduler sees (fixed: batch)
   long long rows;    // batch * tokens
-  int n_q_max, n_kv_max, n_tt;
+  int n_q_max, n_kv_max;
 };
 
 int check_problem(const sba_problem* p, bool fixed, Sizes* sz) {
@@ -40,12 +40,21 @@ int check_problem(const sba_problem* p, bool fixed, Sizes* sz) {
   sz->rows = (long long)p->batch * p->tokens;
   sz->n_q_max = (int)(sz->rows / BM) + sz->n_docs + 1;
   sz->n_kv_max = (int)(sz->rows / BKV) + sz->n_docs + 1;
-  sz->n_tt = cdiv_i(p->max_doc_len > 0 ? p->max_doc_len : 1, BT);
   return 0;
 }
 
+// Carry-table entries per head.  Fixed-length: exact.  Packed documents: the most any split of
+// `tokens` tokens into documents of at most max_doc_len tokens can need (the per-document need is
+// convex in the length, so the worst split is as many longest documents as fit plus the rest).
+long long table_entries_bound(const sba_problem* p, bool fixed) {
+  if (fixed) return (long long)p->batch * tab_doc_entries(p->tokens);
+  const int lmax = (p->max_doc_len > 0 && p->max_doc_len < p->tokens) ? p->max_doc_len : p->tokens;
+  if (lmax <= 0) return 0;
+  return (long long)(p->tokens / lmax) * tab_doc_entries(lmax) + tab_doc_entries(p->tokens % lmax);
+}
+
 size_t schedule_bytes(const Sizes& sz) {
-  size_t words = SCHED_HDR + 4 * ((size_t)sz.n_q_max + sz.n_kv_max) + 5 * (size_t)sz.n_docs + 2;
+  size_t words = SCHED_HDR + TILE_WORDS * ((size_t)sz.n_q_max + sz.n_kv_max) + 6 * (size_t)sz.n_docs + 2;
   return (words * sizeof(int) + 255) & ~(size_t)255;
 }
 
@@ -109,35 +118,46 @@ struct Timer {
   }
 };
 
-int fill_common(const sba_problem* p, const Sizes& sz, const void* schedule, KArgs* a) {
+// `table_bytes`: size of EACH carry table handed in (ignored when none is).
+int fill_common(const sba_problem* p, bool fixed, const Sizes& sz, const void* schedule, size_t sched_bytes,
+                bool with_table, size_t table_bytes, KArgs* a) {
   if (schedule == nullptr) return SBA_E_NULL;
   if (reinterpret_cast<uintptr_t>(schedule) & 15) return SBA_E_STRIDE;   // kernels read the header as one 16-byte word
+  if (sched_bytes < schedule_bytes(sz)) return SBA_E_WORKSPACE;
+  a->tab_stride = -1;
+  if (with_table) {
+    a->tab_stride = (int64_t)(table_bytes / sizeof(float) / (size_t)p->heads);
+    // fixed-length needs are known here; packed documents are checked on the device against
+    // what the scheduler found (kernels refuse to run, outputs are filled with NaN)
+    if (fixed && a->tab_stride < table_entries_bound(p, true)) return SBA_E_WORKSPACE;
+    if (a->tab_stride <= 0) return SBA_E_WORKSPACE;
+  }
   a->sched = reinterpret_cast<const int*>(schedule);
-  a->kv_list_off = SCHED_HDR + 4 * sz.n_q_max;
+  a->kv_list_off = SCHED_HDR + TILE_WORDS * sz.n_q_max;
   a->heads = p->heads;
   a->tokens = p->tokens;
-  a->n_tt = sz.n_tt;
-  a->n_pl = sz.n_tt + 1;
   a->fuse = (p->flags & SBA_FUSE_REMAINDER) ? 1 : 0;
-  a->rows_total = sz.rows;
   a->inv_temp = p->inv_temp;
   a->c = p->inv_temp * 1.4426950408889634f;
   return 0;
 }
 
-int forward(const sba_problem* p, bool fixed, const void* schedule, const sba_view* q, const sba_view* k,
-            const sba_view* v, const sba_view* o, const sba_view* rem, float* stick, float* weights, void* stream,
-            bool timed = true) {
+int forward(const sba_problem* p, bool fixed, const void* schedule, size_t sched_bytes, const sba_view* q,
+            const sba_view* k, const sba_view* v, const sba_view* o, const sba_view* rem, float* stick,
+            size_t table_bytes, float* weights, size_t weights_bytes, void* stream, bool timed = true) {
   Sizes sz;
   int e = check_problem(p, fixed, &sz);
   if (e) return e;
   if ((e = check_mat(q, p)) || (e = check_mat(k, p)) || (e = check_mat(v, p)) || (e = check_mat(o, p))) return e;
   if ((e = check_view(rem, true))) return e;
-  if ((e = check_arch())) return e;
-  if (sz.rows == 0) return 0;
+  if (weights != nullptr &&
+      weights_bytes / sizeof(float) < (size_t)p->batch * p->heads * (size_t)p->tokens * (size_t)p->tokens)
+    return SBA_E_WORKSPACE;
   KArgs a;
   std::memset(&a, 0, sizeof(a));
-  if ((e = fill_common(p, sz, schedule, &a))) return e;
+  if ((e = fill_common(p, fixed, sz, schedule, sched_bytes, stick != nullptr, table_bytes, &a))) return e;
+  if ((e = check_arch())) return e;
+  if (sz.rows == 0) return 0;
   a.q = to_view(q); a.k = to_view(k); a.v = to_view(v); a.o = to_view(o); a.rem = to_view(rem);
   a.stick = stick;
   a.weights = weights;
@@ -153,12 +173,14 @@ int forward(const sba_problem* p, bool fixed, const void* schedule, const sba_vi
   std::memset(&z, 0, sizeof(z));
   z.mat[0] = a.o; z.n_mat = 1; z.row = a.rem;
   z.sched = a.sched; z.heads = p->heads; z.tokens = p->tokens; z.head_dim = p->head_dim;
+  z.tab_stride = a.tab_stride;
   return (int)launch_zero_tail(z, s);
 }
 
-int backward(const sba_problem* p, bool fixed, const void* schedule, const sba_view* q, const sba_view* k,
-             const sba_view* v, const sba_view* go, const sba_view* grem, const float* stick, float* gtab,
-             const sba_view* dq, const sba_view* dk, const sba_view* dv, void* stream) {
+int backward(const sba_problem* p, bool fixed, const void* schedule, size_t sched_bytes, const sba_view* q,
+             const sba_view* k, const sba_view* v, const sba_view* go, const sba_view* grem, const float* stick,
+             float* gtab, size_t table_bytes, const sba_view* dq, const sba_view* dk, const sba_view* dv,
+             void* stream) {
   Sizes sz;
   int e = check_problem(p, fixed, &sz);
   if (e) return e;
@@ -166,11 +188,11 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, const sba_v
       (e = check_mat(dq, p)) || (e = check_mat(dk, p)) || (e = check_mat(dv, p)))
     return e;
   if (stick == nullptr || gtab == nullptr) return SBA_E_NULL;
-  if ((e = check_arch())) return e;
-  if (sz.rows == 0) return 0;
   KArgs a;
   std::memset(&a, 0, sizeof(a));
-  if ((e = fill_common(p, sz, schedule, &a))) return e;
+  if ((e = fill_common(p, fixed, sz, schedule, sched_bytes, true, table_bytes, &a))) return e;
+  if ((e = check_arch())) return e;
+  if (sz.rows == 0) return 0;
   a.q = to_view(q); a.k = to_view(k); a.v = to_view(v); a.go = to_view(go);
   a.grem = to_view(grem);
   a.dq = to_view(dq); a.dk = to_view(dk); a.dv = to_view(dv);
@@ -195,6 +217,7 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, const sba_v
   std::memset(&z, 0, sizeof(z));
   z.mat[0] = a.dq; z.mat[1] = a.dk; z.mat[2] = a.dv; z.n_mat = 3;
   z.sched = a.sched; z.heads = p->heads; z.tokens = p->tokens; z.head_dim = p->head_dim;
+  z.tab_stride = a.tab_stride;
   return (int)launch_zero_tail(z, s);
 }
 
@@ -254,66 +277,86 @@ size_t sba_table_bytes(const sba_problem* p) {
   Sizes sz;
   const bool fixed = p != nullptr && (p->flags & SBA_FIXED_LENGTH) != 0;
   if (check_problem(p, fixed, &sz)) return 0;
-  return (size_t)p->heads * ((size_t)sz.n_tt + 1) * (size_t)sz.rows * sizeof(float);
+  return (size_t)p->heads * (size_t)table_entries_bound(p, fixed) * sizeof(float);
 }
 
-int sba_build_schedule(const sba_problem* p, void* schedule, void* stream) {
+size_t sba_table_bytes_for_lengths(const sba_problem* p, const int64_t* doc_lengths, int n_lengths) {
+  Sizes sz;
+  const bool fixed = p != nullptr && (p->flags & SBA_FIXED_LENGTH) != 0;
+  if (check_problem(p, fixed, &sz) || (n_lengths > 0 && doc_lengths == nullptr)) return 0;
+  if (fixed) return sba_table_bytes(p);
+  long long entries = 0;
+  for (int i = 0; i < n_lengths; ++i) {
+    if (doc_lengths[i] < 0 || doc_lengths[i] > p->tokens) return 0;
+    entries += tab_doc_entries((int)doc_lengths[i]);
+  }
+  if (entries > 0x7fffffffll) return 0;   // a document's base must fit the scheduler's int32 field
+  return (size_t)p->heads * (size_t)(entries > 0 ? entries : 1) * sizeof(float);
+}
+
+int sba_build_schedule(const sba_problem* p, void* schedule, size_t schedule_size, void* stream) {
   Sizes sz;
   const bool fixed = p != nullptr && (p->flags & SBA_FIXED_LENGTH) != 0;
   int e = check_problem(p, fixed, &sz);
   if (e) return e;
   if (schedule == nullptr) return SBA_E_NULL;
+  if (schedule_size < schedule_bytes(sz)) return SBA_E_WORKSPACE;
   if ((e = check_arch())) return e;
   SchedArgs a;
   a.cu = fixed ? nullptr : p->cu_seqlens;
   a.cu_is64 = (p->flags & SBA_CU_INT64) ? 1 : 0;
   a.n_docs = sz.n_docs;
   a.tokens = p->tokens;
-  a.max_doc_len = p->max_doc_len;
   a.n_q_max = sz.n_q_max;
   a.n_kv_max = sz.n_kv_max;
   a.out = reinterpret_cast<int*>(schedule);
   return (int)launch_schedule(a, reinterpret_cast<hipStream_t>(stream));
 }
 
-int sba_varlen_fwd(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
-                   const sba_view* v, const sba_view* o, const sba_view* rem, float* stick_table,
-                   void* stream) {
-  return forward(p, false, schedule, q, k, v, o, rem, stick_table, nullptr, stream);
+int sba_varlen_fwd(const sba_problem* p, const void* schedule, size_t schedule_size, const sba_view* q,
+                   const sba_view* k, const sba_view* v, const sba_view* o, const sba_view* rem,
+                   float* stick_table, size_t table_size, void* stream) {
+  return forward(p, false, schedule, schedule_size, q, k, v, o, rem, stick_table, table_size, nullptr, 0, stream);
 }
 
-int sba_attn_fwd(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
-                 const sba_view* v, const sba_view* o, const sba_view* rem, float* stick_table,
-                 void* stream) {
-  return forward(p, true, schedule, q, k, v, o, rem, stick_table, nullptr, stream);
+int sba_attn_fwd(const sba_problem* p, const void* schedule, size_t schedule_size, const sba_view* q,
+                 const sba_view* k, const sba_view* v, const sba_view* o, const sba_view* rem,
+                 float* stick_table, size_t table_size, void* stream) {
+  return forward(p, true, schedule, schedule_size, q, k, v, o, rem, stick_table, table_size, nullptr, 0, stream);
 }
 
-int sba_varlen_fwd_weights(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
-                           const sba_view* v, const sba_view* o, const sba_view* rem, float* stick_table,
-                           float* weights, void* stream) {
+int sba_varlen_fwd_weights(const sba_problem* p, const void* schedule, size_t schedule_size, const sba_view* q,
+                           const sba_view* k, const sba_view* v, const sba_view* o, const sba_view* rem,
+                           float* stick_table, size_t table_size, float* weights, size_t weights_size,
+                           void* stream) {
   if (weights == nullptr) return SBA_E_NULL;
-  return forward(p, false, schedule, q, k, v, o, rem, stick_table, weights, stream);
+  return forward(p, false, schedule, schedule_size, q, k, v, o, rem, stick_table, table_size, weights, weights_size,
+                 stream);
 }
 
-int sba_attn_fwd_weights(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
-                         const sba_view* v, const sba_view* o, const sba_view* rem, float* stick_table,
-                         float* weights, void* stream) {
+int sba_attn_fwd_weights(const sba_problem* p, const void* schedule, size_t schedule_size, const sba_view* q,
+                         const sba_view* k, const sba_view* v, const sba_view* o, const sba_view* rem,
+                         float* stick_table, size_t table_size, float* weights, size_t weights_size,
+                         void* stream) {
   if (weights == nullptr) return SBA_E_NULL;
-  return forward(p, true, schedule, q, k, v, o, rem, stick_table, weights, stream);
+  return forward(p, true, schedule, schedule_size, q, k, v, o, rem, stick_table, table_size, weights, weights_size,
+                 stream);
 }
 
-int sba_varlen_bwd(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
-                   const sba_view* v, const sba_view* grad_o, const sba_view* grad_rem,
-                   const float* stick_table, float* grad_table, const sba_view* dq, const sba_view* dk,
-                   const sba_view* dv, void* stream) {
-  return backward(p, false, schedule, q, k, v, grad_o, grad_rem, stick_table, grad_table, dq, dk, dv, stream);
+int sba_varlen_bwd(const sba_problem* p, const void* schedule, size_t schedule_size, const sba_view* q,
+                   const sba_view* k, const sba_view* v, const sba_view* grad_o, const sba_view* grad_rem,
+                   const float* stick_table, float* grad_table, size_t table_size, const sba_view* dq,
+                   const sba_view* dk, const sba_view* dv, void* stream) {
+  return backward(p, false, schedule, schedule_size, q, k, v, grad_o, grad_rem, stick_table, grad_table, table_size,
+                  dq, dk, dv, stream);
 }
 
-int sba_attn_bwd(const sba_problem* p, const void* schedule, const sba_view* q, const sba_view* k,
-                 const sba_view* v, const sba_view* grad_o, const sba_view* grad_rem,
-                 const float* stick_table, float* grad_table, const sba_view* dq, const sba_view* dk,
-                 const sba_view* dv, void* stream) {
-  return backward(p, true, schedule, q, k, v, grad_o, grad_rem, stick_table, grad_table, dq, dk, dv, stream);
+int sba_attn_bwd(const sba_problem* p, const void* schedule, size_t schedule_size, const sba_view* q,
+                 const sba_view* k, const sba_view* v, const sba_view* grad_o, const sba_view* grad_rem,
+                 const float* stick_table, float* grad_table, size_t table_size, const sba_view* dq,
+                 const sba_view* dk, const sba_view* dv, void* stream) {
+  return backward(p, true, schedule, schedule_size, q, k, v, grad_o, grad_rem, stick_table, grad_table, table_size,
+                  dq, dk, dv, stream);
 }
 
 int sba_varlen_fwd_static(const sba_problem* p, const sba_view* q, const sba_view* k, const sba_view* v,
@@ -327,8 +370,9 @@ int sba_varlen_fwd_static(const sba_problem* p, const sba_view* q, const sba_vie
   if ((e = static_scratch(&sched))) return e;
   // The scheduler rewrites the header and every list entry the kernels will use; nothing of
   // the previous call's contents is read, so nothing needs clearing.
-  if ((e = sba_build_schedule(p, sched, stream))) return e;
-  return forward(p, false, sched, q, k, v, o, rem, nullptr, nullptr, stream, /*timed=*/false);   // (timing creates events)
+  if ((e = sba_build_schedule(p, sched, SBA_STATIC_SCRATCH_BYTES, stream))) return e;
+  return forward(p, false, sched, SBA_STATIC_SCRATCH_BYTES, q, k, v, o, rem, nullptr, 0, nullptr, 0, stream,
+                 /*timed=*/false);   // (timing creates events)
 }
 
 void sba_set_timing(int on) { g_timing.store(on); }

@@ -114,10 +114,10 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   const int* sched = a.sched;
   const int slot = blockIdx.x / a.heads;
   const int head = blockIdx.x - slot * a.heads;
-  const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, longest document
+  const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, table entries needed
   const Tile t = reinterpret_cast<const Tile*>(sched + SCHED_HDR)[slot];
-  asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch));   // keep the tile read above the branch
-  if (hdr.x != 0 || slot >= hdr.y) return;
+  asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch), "s"(t.tab_base));   // keep the tile read above the branch
+  if (hdr.x != 0 || slot >= hdr.y || hdr.w > a.tab_stride) return;
 
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -133,7 +133,6 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   const __bf16* vb = reinterpret_cast<const __bf16*>(a.v.ptr) + t.batch * a.v.sb + head * a.v.sh + tok0 * a.v.st;
   const __bf16* gob = reinterpret_cast<const __bf16*>(a.go.ptr) + t.batch * a.go.sb + head * a.go.sh + tok0 * a.go.st;
   __bf16* dqb = reinterpret_cast<__bf16*>(a.dq.ptr) + t.batch * a.dq.sb + head * a.dq.sh + tok0 * a.dq.st;
-  const int64_t grow = (int64_t)t.batch * a.tokens + tok0 + qrow;
   const Rows qrows = make_rows(qb, a.q.st, t.doc_len);
   const Rows grows = make_rows(gob, a.go.st, t.doc_len);
   const Rows krows = make_rows(kb, a.k.st, t.doc_len);
@@ -195,18 +194,18 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
       toff[u][db] = swz_off<D>(r, col >> 3) + (col & 7);
     }
   }
-  const int64_t tab0 = (int64_t)head * a.n_pl * a.rows_total + grow;
+  const int64_t tab0 = (int64_t)head * a.tab_stride + t.tab_base + qrow;   // this row's entries of the document's table area
   const float* stick = a.stick + tab0;
   float* gtab = a.gtab + tab0;
   // the dk/dv pass takes d(rem) from the last plane of the gradient table
-  if (qvalid && h == 0) gtab[(int64_t)a.n_tt * a.rows_total] = dr;
+  if (qvalid && h == 0) gtab[tab_rowplane(t.doc_len)] = dr;
 
   // stick carries of the two sub-blocks of a tile (neutral where the sub-block is skipped)
   auto carries = [&](int kt, float (&ce)[2]) {
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
       ce[sb] = PROD ? 1.0f : 0.0f;
-      if (qvalid && kt <= kt_last && !sub_skip<AC>(kt * BN + 32 * sb, qw0)) ce[sb] = stick[(int64_t)(2 * kt + sb) * a.rows_total];
+      if (qvalid && kt <= kt_last && !sub_skip<AC>(kt * BN + 32 * sb, qw0)) ce[sb] = stick[tab_seg(t.doc_len, 2 * kt + sb)];
     }
   };
   float ce[2], ce_next[2];
@@ -231,7 +230,7 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
     for (int sb = 0; sb < 2; ++sb) {
       const int k0 = kt * BN + 32 * sb;
       if (sub_skip<AC>(k0, qw0)) continue;
-      const int64_t tix = (int64_t)(2 * kt + sb) * a.rows_total;
+      const int64_t tix = tab_seg(t.doc_len, 2 * kt + sb);
       if (qvalid && h == 0) gtab[tix] = carry_c;
       // LDS latency under load is several hundred cycles, so every group of operand reads is
       // issued one phase before the MFMAs that consume it: V rows before the weights are
@@ -328,10 +327,10 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   const int* sched = a.sched;
   const int slot = blockIdx.x / a.heads;
   const int head = blockIdx.x - slot * a.heads;
-  const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, longest document
+  const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, table entries needed
   const Tile t = reinterpret_cast<const Tile*>(sched + a.kv_list_off)[slot];
-  asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch));   // keep the tile read above the branch
-  if (hdr.x != 0 || slot >= hdr.z) return;
+  asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch), "s"(t.tab_base));   // keep the tile read above the branch
+  if (hdr.x != 0 || slot >= hdr.z || hdr.w > a.tab_stride) return;
   const int kt = t.idx;
 
   const int tid = threadIdx.x;
@@ -370,12 +369,13 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       vf[ks] = load_frag(vrows, k0 + kperm(n), 32 * ks + 16 * h);
     }
     // A block that starts past the end of the document is never visible to a query; its table
-    // reads are redirected to the document's last block so that they stay inside the tables
-    // (which hold ceil(max_doc_len / 32) blocks per row), and their values are never used.
+    // reads are redirected to the document's last block so that they stay inside the document's
+    // table area, and their values are never used.  (Rows above a block's first row, read by the
+    // first steps of the later blocks, fall into the preceding block's rows: in bounds, unused.)
     const int tblock = min((BKV / 32) * kt + sb, (t.doc_len - 1) / 32);
-    const int64_t tab_row0 = (int64_t)head * a.n_pl * a.rows_total + (int64_t)t.batch * a.tokens + tok0;
-    const int64_t tab = tab_row0 + (int64_t)tblock * a.rows_total;
-    const int64_t tab_rowval = tab_row0 + (int64_t)a.n_tt * a.rows_total;   // per-row plane: rem (stick table), d(rem) (gradient table, written by the dq pass)
+    const int64_t tab_row0 = (int64_t)head * a.tab_stride + t.tab_base;
+    const int64_t tab = tab_row0 + tab_seg(t.doc_len, tblock);
+    const int64_t tab_rowval = tab_row0 + tab_rowplane(t.doc_len);   // per-row plane: rem (stick table), d(rem) (gradient table, written by the dq pass)
     // Fused output o + rem * v: its gradient reaches v_j directly as rem_j * do_j.  The queries of
     // step `sb` are this wave's own keys, so that term is dv = P^T dO with rem_j added on the
     // diagonal of P (which is otherwise zero, or p_jj with attend_current), at no extra traffic.

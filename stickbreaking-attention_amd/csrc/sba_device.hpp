@@ -31,16 +31,30 @@ constexpr int NT = 256;  // threads per workgroup
 constexpr int SCHED_STATUS = 0;
 constexpr int SCHED_NQ = 1;      // number of query tiles
 constexpr int SCHED_NKV = 2;     // number of KV tiles
-constexpr int SCHED_MAXLEN = 3;  // longest document found
+constexpr int SCHED_TABLE = 3;   // carry-table entries per head the documents need (saturates at INT_MAX)
 constexpr int SCHED_TOTAL = 4;   // tokens covered by the documents (0 when the input is rejected)
+constexpr int SCHED_MAXLEN = 5;  // longest document found
 constexpr int SCHED_HDR = 16;    // tile lists start here
+constexpr int TILE_WORDS = 8;    // int32 words of one Tile
 
 struct Tile {
   int tok_start;  // first token of the document inside the packed token axis (0 for fixed-length)
   int doc_len;
   int idx;        // tile index inside the document
   int batch;      // batch entry (0 for varlen)
+  int tab_base;   // first carry-table entry of the document inside a head's share of the tables
+  int rsv[3];
 };
+
+// Carry tables (fp32).  Inside a head's share every document owns a triangular area: for each
+// 32-key block b the rows 32*b .. L-1 (the queries at or below the block), blocks back to back,
+// then one plane of L per-row values.  Entry (b, row) sits at  tab_seg(L, b) + row  from the
+// document's base: consecutive rows are consecutive floats, so the 32 lanes that own 32
+// consecutive query rows read and write 128 contiguous bytes.
+__host__ __device__ inline long long tab_block_off(int L, int b) { return (long long)b * L - 16ll * b * (b - 1); }
+__host__ __device__ inline long long tab_seg(int L, int b) { return tab_block_off(L, b) - 32ll * b; }
+__host__ __device__ inline long long tab_rowplane(int L) { return tab_block_off(L, (L + 31) / 32); }
+__host__ __device__ inline long long tab_doc_entries(int L) { return tab_rowplane(L) + L; }
 
 struct View {
   char* ptr;

@@ -31,10 +31,10 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   const int* sched = a.sched;
   const int slot = blockIdx.x / a.heads;
   const int head = blockIdx.x - slot * a.heads;
-  const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, longest document
+  const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, table entries needed
   const Tile t = reinterpret_cast<const Tile*>(sched + SCHED_HDR)[slot];
   asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch));   // keep the tile read above the branch
-  if (hdr.x != 0 || slot >= hdr.y) return;
+  if (hdr.x != 0 || slot >= hdr.y || (a.stick != nullptr && hdr.w > a.tab_stride)) return;
 
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -50,7 +50,6 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   const __bf16* vb = reinterpret_cast<const __bf16*>(a.v.ptr) + t.batch * a.v.sb + head * a.v.sh + tok0 * a.v.st;
   __bf16* ob = reinterpret_cast<__bf16*>(a.o.ptr) + t.batch * a.o.sb + head * a.o.sh + tok0 * a.o.st;
   __bf16* rb = reinterpret_cast<__bf16*>(a.rem.ptr) + t.batch * a.rem.sb + head * a.rem.sh + tok0 * a.rem.st;
-  const int64_t grow = (int64_t)t.batch * a.tokens + tok0 + qrow;  // row index in the tables
   const Rows qrows = make_rows(qb, a.q.st, t.doc_len);
   const Rows krows = make_rows(kb, a.k.st, t.doc_len);
   const Rows vrows = make_rows(vb, a.v.st, t.doc_len);
@@ -97,7 +96,8 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
       voff[u][db] = swz_off<D>(r, col >> 3) + (col & 7);
     }
   }
-  float* stick = a.stick == nullptr ? nullptr : a.stick + (int64_t)head * a.n_pl * a.rows_total + grow;
+  // this row's entries of the document's triangular table area
+  float* stick = a.stick == nullptr ? nullptr : a.stick + (int64_t)head * a.tab_stride + t.tab_base + qrow;
 
   // One tile step; the ring slot is a compile-time constant so every LDS address is a fixed
   // register plus an immediate.
@@ -117,7 +117,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
     const int k0 = kt * BF;
     if (sub_skip<AC>(k0, qw0)) return;
     // stick left on entering this block: what both backward kernels start it from
-    if (stick != nullptr && h == 0 && qvalid) stick[(int64_t)kt * a.rows_total] = carry;
+    if (stick != nullptr && h == 0 && qvalid) stick[tab_seg(t.doc_len, kt)] = carry;
     f32x16 x;
 #pragma unroll
     for (int i = 0; i < 16; ++i) x[i] = 0.0f;
@@ -179,7 +179,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   if (h == 0 && qvalid) {
     rb[(int64_t)qrow * a.rem.st] = (__bf16)r;
     // rem in full precision for the backward of the fused output (last plane of the table)
-    if (stick != nullptr) stick[(int64_t)a.n_tt * a.rows_total] = r;
+    if (stick != nullptr) stick[tab_rowplane(t.doc_len)] = r;
   }
   lds_barrier();   // every wave is done with the K/V tiles: their memory becomes the o staging area
   if (a.fuse) {

@@ -12,17 +12,15 @@ struct KArgs {
   View go, grem, dq, dk, dv;   // backward tensors (grem.ptr may be null)
   const int* sched;            // schedule workspace
   int kv_list_off;             // int32 offset of the KV tile list inside `sched`
-  float* stick;                // carry table written by the forward (may be null in fwd)
-  float* gtab;                 // gradient prefix table (backward scratch)
+  float* stick;                // carry table written by the forward (may be null in fwd): per (row, 32-key block) the
+                               // stick left on entering the block; per-row plane: rem in fp32
+  float* gtab;                 // gradient prefix table (backward scratch); per-row plane: the full d(rem)
   float* weights;              // forward, debug variant only: dense attention weights
                                // [batch][heads][tokens][tokens] (row = query token, column = key token)
   int heads;
   int tokens;                  // tokens per batch entry
-  int n_tt;                    // table blocks per row = ceil(max_doc_len / 32)
-  int n_pl;                    // planes of a table = n_tt + 1; the last one holds per-row values
-                               // (stick table: rem in fp32; gradient table: the full d(rem))
   int fuse;                    // the output is o + rem * v (and grad_o is the gradient of that)
-  int64_t rows_total;          // batch * tokens
+  int64_t tab_stride;          // carry-table entries per head the caller's tables hold
   float c;                     // inv_temp * log2(e)
   float inv_temp;
 };
@@ -32,7 +30,6 @@ struct SchedArgs {
   int cu_is64;
   int n_docs;       // documents (fixed: batch)
   int tokens;       // T per batch entry
-  int max_doc_len;
   int n_q_max, n_kv_max;
   int* out;
 };
@@ -44,6 +41,7 @@ struct ZeroArgs {
   View row;         // per-row output (rem); ptr may be null
   const int* sched;
   int heads, tokens, head_dim;
+  int64_t tab_stride;   // table entries per head available to the launch that wrote these outputs (< 0: no table in use)
 };
 
 hipError_t launch_schedule(const SchedArgs& a, hipStream_t s);

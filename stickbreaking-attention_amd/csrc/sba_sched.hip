@@ -15,10 +15,11 @@ constexpr int RANK_LIMIT = 4096;   // beyond this many documents the input order
 
 __device__ __forceinline__ int cdiv(int a, int b) { return (a + b - 1) / b; }
 
-// Scratch (int32) behind the two tile lists, per document: start, len, order, qoff, kvoff.
+// Scratch (int32) behind the two tile lists, per document: start, len, order, qoff, kvoff, table base.
 __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a) {
   __shared__ int s_status, s_maxlen;
   __shared__ int s_scan_q[SCHED_THREADS], s_scan_kv[SCHED_THREADS];
+  __shared__ long long s_scan_tab[SCHED_THREADS];
   const int tid = threadIdx.x;
   const int nd = a.n_docs;
   int* hdr = a.out;
@@ -29,6 +30,7 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
   int* order = dlen + nd;
   int* qoff = order + nd;         // nd + 1 entries
   int* kvoff = qoff + nd + 1;     // nd + 1 entries
+  int* dtab = kvoff + nd + 1;     // first carry-table entry of each document (by document index)
   const bool fixed = a.cu == nullptr;
 
   if (tid == 0) { s_status = 0; s_maxlen = 0; }
@@ -52,7 +54,6 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
       st = 0;
     } else {
       len = (int)(en - st);
-      if (len > a.max_doc_len) atomicOr(&s_status, 2);   // SBA_STATUS_DOC_TOO_LONG
     }
     dstart[d] = (int)st;
     dlen[d] = len;
@@ -78,33 +79,45 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
   // C. exclusive prefix of the tile counts in ranked order
   const int per = cdiv(nd, SCHED_THREADS);
   int sq = 0, skv = 0;
+  long long stab = 0;
   for (int j = 0; j < per; ++j) {
     const int i = tid * per + j;
     if (i < nd) {
       const int len = dlen[order[i]];
       sq += cdiv(len, BM);
       skv += cdiv(len, BKV);
+      stab += tab_doc_entries(len);
     }
   }
   s_scan_q[tid] = sq;
   s_scan_kv[tid] = skv;
+  s_scan_tab[tid] = stab;
   __syncthreads();
   for (int off = 1; off < SCHED_THREADS; off <<= 1) {
     int vq = 0, vkv = 0;
-    if (tid >= off) { vq = s_scan_q[tid - off]; vkv = s_scan_kv[tid - off]; }
+    long long vtab = 0;
+    if (tid >= off) { vq = s_scan_q[tid - off]; vkv = s_scan_kv[tid - off]; vtab = s_scan_tab[tid - off]; }
     __syncthreads();
     s_scan_q[tid] += vq;
     s_scan_kv[tid] += vkv;
+    s_scan_tab[tid] += vtab;
     __syncthreads();
   }
   int bq = s_scan_q[tid] - sq, bkv = s_scan_kv[tid] - skv;
+  long long btab = s_scan_tab[tid] - stab;
+  const long long total_tab = s_scan_tab[SCHED_THREADS - 1];
+  // a document's table base must fit an int32 tile field; larger totals are reported through the
+  // saturated header word and refused by every kernel that uses a table
+  const bool tab_ok = total_tab <= 0x7fffffffll;
   for (int j = 0; j < per; ++j) {
     const int i = tid * per + j;
     if (i < nd) {
       const int len = dlen[order[i]];
       qoff[i] = bq; kvoff[i] = bkv;
+      dtab[order[i]] = tab_ok ? (int)btab : 0;
       bq += cdiv(len, BM);
       bkv += cdiv(len, BKV);
+      btab += tab_doc_entries(len);
     }
   }
   const int total_q = s_scan_q[SCHED_THREADS - 1], total_kv = s_scan_kv[SCHED_THREADS - 1];
@@ -137,6 +150,8 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
     t.doc_len = dlen[d];
     t.idx = nq - 1 - within;             // newest (most expensive) query tile first
     t.batch = fixed ? d : 0;
+    t.tab_base = dtab[d];
+    t.rsv[0] = t.rsv[1] = t.rsv[2] = 0;
     qtiles[s] = t;
   }
   // Key tiles stay document-major for every input: one workgroup per CU runs at a time, so the
@@ -151,6 +166,8 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
     t.doc_len = dlen[d];
     t.idx = s - kvoff[lo];               // oldest keys are seen by the most queries: first
     t.batch = fixed ? d : 0;
+    t.tab_base = dtab[d];
+    t.rsv[0] = t.rsv[1] = t.rsv[2] = 0;
     kvtiles[s] = t;
   }
   if (tid == 0) {
@@ -158,6 +175,7 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
     hdr[SCHED_NQ] = ok ? total_q : 0;
     hdr[SCHED_NKV] = ok ? total_kv : 0;
     hdr[SCHED_MAXLEN] = s_maxlen;
+    hdr[SCHED_TABLE] = tab_ok ? (int)total_tab : 0x7fffffff;
     hdr[SCHED_TOTAL] = (ok && nd > 0) ? dstart[nd - 1] + dlen[nd - 1] : 0;
   }
 }
@@ -166,16 +184,19 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
 // (empty_like, sb_varlen_fwd.py:418) and relies on zeros_like elsewhere (sb_varlen_bwd.py:507-509).
 // Here the compute kernels write every row of every document exactly once, so only the rows
 // that belong to no document need clearing: 64 rows per workgroup, which exits at once when
-// its rows are covered.  When the schedule was rejected (malformed cu_seqlens) nothing else
-// runs and everything is cleared.
+// its rows are covered.  When nothing else ran -- the scheduler rejected cu_seqlens, or the
+// carry tables handed in are smaller than the documents need -- every row is filled with NaN
+// instead, so that the failure cannot pass for a result.
 constexpr int ZERO_ROWS = 64;
 __global__ void __launch_bounds__(256) zero_tail_kernel(const ZeroArgs a) {
-  const int total = a.sched[SCHED_TOTAL];
+  const bool refused = a.sched[SCHED_STATUS] != 0 || (a.tab_stride >= 0 && a.sched[SCHED_TABLE] > a.tab_stride);
+  const int total = refused ? 0 : a.sched[SCHED_TOTAL];
   const int row0 = blockIdx.x * ZERO_ROWS;
   const int lo = max(row0, total), hi = min(row0 + ZERO_ROWS, a.tokens);
   if (lo >= hi) return;
   const int nrows = hi - lo, c8 = a.head_dim / 8;
-  const uint4 z = make_uint4(0u, 0u, 0u, 0u);
+  const unsigned fill = refused ? 0x7fc07fc0u : 0u;   // two bf16 NaNs, or zeros
+  const uint4 z = make_uint4(fill, fill, fill, fill);
   for (int head = 0; head < a.heads; ++head) {
     for (int m = 0; m < a.n_mat; ++m) {
       unsigned short* base = reinterpret_cast<unsigned short*>(a.mat[m].ptr) + head * a.mat[m].sh + lo * a.mat[m].st;
@@ -184,7 +205,7 @@ __global__ void __launch_bounds__(256) zero_tail_kernel(const ZeroArgs a) {
     }
     if (a.row.ptr != nullptr) {
       unsigned short* base = reinterpret_cast<unsigned short*>(a.row.ptr) + head * a.row.sh + lo * a.row.st;
-      for (int r = threadIdx.x; r < nrows; r += 256) base[r * a.row.st] = 0;
+      for (int r = threadIdx.x; r < nrows; r += 256) base[r * a.row.st] = (unsigned short)fill;
     }
   }
 }

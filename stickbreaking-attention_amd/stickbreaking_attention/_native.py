@@ -25,8 +25,7 @@ FLAG_FUSE_REMAINDER = 16
 
 STATUS_MESSAGES = {
     1: "cu_seqlens is not a non-decreasing sequence within [0, total_tokens]",
-    2: "a document is longer than max_seqlens",
-    3: "cu_seqlens is invalid and a document is longer than max_seqlens",
+    4: "the carry tables are too small for the documents in cu_seqlens (max_seqlens under-states a document)",
 }
 
 
@@ -43,7 +42,8 @@ class SbaProblem(ctypes.Structure):
 
 
 EXPORTS = (
-    "sba_version", "sba_error_string", "sba_schedule_bytes", "sba_table_bytes", "sba_build_schedule",
+    "sba_version", "sba_error_string", "sba_schedule_bytes", "sba_table_bytes", "sba_table_bytes_for_lengths",
+    "sba_build_schedule",
     "sba_varlen_fwd", "sba_varlen_bwd", "sba_attn_fwd", "sba_attn_bwd", "sba_set_timing",
     "sba_last_kernel_ms", "sba_varlen_fwd_weights", "sba_attn_fwd_weights", "sba_varlen_fwd_static",
 )
@@ -73,20 +73,23 @@ def load():
         lib.sba_schedule_bytes.argtypes = [P]
         lib.sba_table_bytes.restype = ctypes.c_size_t
         lib.sba_table_bytes.argtypes = [P]
+        sz = ctypes.c_size_t
+        lib.sba_table_bytes_for_lengths.restype = ctypes.c_size_t
+        lib.sba_table_bytes_for_lengths.argtypes = [P, ctypes.POINTER(ctypes.c_int64), ctypes.c_int]
         lib.sba_build_schedule.restype = ctypes.c_int
-        lib.sba_build_schedule.argtypes = [P, vp, vp]
+        lib.sba_build_schedule.argtypes = [P, vp, sz, vp]
         for name in ("sba_varlen_fwd", "sba_attn_fwd"):
             f = getattr(lib, name)
             f.restype = ctypes.c_int
-            f.argtypes = [P, vp, V, V, V, V, V, vp, vp]
+            f.argtypes = [P, vp, sz, V, V, V, V, V, vp, sz, vp]
         for name in ("sba_varlen_fwd_weights", "sba_attn_fwd_weights"):
             f = getattr(lib, name)
             f.restype = ctypes.c_int
-            f.argtypes = [P, vp, V, V, V, V, V, vp, vp, vp]
+            f.argtypes = [P, vp, sz, V, V, V, V, V, vp, sz, vp, sz, vp]
         for name in ("sba_varlen_bwd", "sba_attn_bwd"):
             f = getattr(lib, name)
             f.restype = ctypes.c_int
-            f.argtypes = [P, vp, V, V, V, V, V, vp, vp, V, V, V, vp]
+            f.argtypes = [P, vp, sz, V, V, V, V, V, vp, vp, sz, V, V, V, vp]
         lib.sba_varlen_fwd_static.restype = ctypes.c_int
         lib.sba_varlen_fwd_static.argtypes = [P, V, V, V, V, V, vp]
         lib.sba_set_timing.restype = None

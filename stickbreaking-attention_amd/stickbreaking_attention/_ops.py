@@ -17,7 +17,8 @@ import ctypes
 import math
 import os
 import warnings
-from typing import Optional, Tuple
+import weakref
+from typing import Optional, Sequence, Tuple
 
 import torch
 
@@ -28,14 +29,21 @@ from .utils import custom_op
 # log2 sum (3 per score).  Overridable for A/B measurements.
 PRODUCT_SPACE = os.environ.get("SBA_LOG_SPACE", "0") != "1"
 
-# When True every eager forward reads back the scheduler's status word (one device sync) and
-# raises on malformed cu_seqlens instead of returning zero outputs.
+# When True every eager forward reads back the scheduler's status words (one device sync) and
+# raises on malformed cu_seqlens or undersized tables instead of returning NaN outputs.
 VALIDATE = os.environ.get("SBA_VALIDATE", "0") == "1"
+
+# Eager calls copy each NEW cu_seqlens tensor to the host once (one synchronisation per tensor
+# object and version; a model hands the same tensor to every layer) so that the carry tables are
+# sized exactly and malformed cu_seqlens raise at once.  With SBA_SYNC_FREE=1 -- and always while
+# torch.compile traces -- nothing is read back: tables get the worst-case size for
+# (tokens, max_seqlens) and errors surface as NaN outputs.
+SYNC_FREE = os.environ.get("SBA_SYNC_FREE", "0") == "1"
 
 SUPPORTED_HEAD_DIMS = (64, 128)
 
 # Tile sizes the library's workspace formulas are built on (query tile, dk/dv key tile, table block).
-_BM, _BKV, _BT, _SCHED_HDR = 128, 128, 32, 16
+_BM, _BKV, _BT, _SCHED_HDR, _TILE_WORDS = 128, 128, 32, 16, 8
 
 
 def _padded_dim(d: int) -> int:
@@ -45,17 +53,101 @@ def _padded_dim(d: int) -> int:
     raise ValueError(f"head_dim {d} is not supported (maximum {SUPPORTED_HEAD_DIMS[-1]})")
 
 
-def workspace_sizes(fixed: bool, batch: int, heads: int, tokens: int, n_docs: int, max_doc_len: int) -> Tuple[int, int]:
+def table_entries(length: int) -> int:
+    """Carry-table entries one document of `length` tokens needs per head: one per (32-key block,
+    query row at or below it) pair plus one per row (``tab_doc_entries`` in csrc/sba_device.hpp)."""
+    nb = -(-length // _BT)
+    return nb * length - 16 * nb * (nb - 1) + length
+
+
+def table_entries_bound(tokens: int, max_doc_len: int) -> int:
+    """The most any split of `tokens` tokens into documents of at most `max_doc_len` can need."""
+    lmax = max_doc_len if 0 < max_doc_len < tokens else tokens
+    if lmax <= 0:
+        return 0
+    return (tokens // lmax) * table_entries(lmax) + table_entries(tokens % lmax)
+
+
+def workspace_sizes(fixed: bool, batch: int, heads: int, tokens: int, n_docs: int, max_doc_len: int,
+                    lengths: Optional[Sequence[int]] = None) -> Tuple[int, int]:
     """(schedule bytes, floats of one carry table): the same numbers as ``sba_schedule_bytes`` and
-    ``sba_table_bytes // 4``, computed without touching the library so that they can be
-    evaluated while a graph is being traced (checked against the library in the tests)."""
+    ``sba_table_bytes // 4`` (``sba_table_bytes_for_lengths // 4`` when the document lengths are
+    given), computed without touching the library so that they can be evaluated while a graph is
+    being traced (checked against the library in the tests)."""
     docs = batch if fixed else n_docs
     rows = (batch if fixed else 1) * tokens
     n_q = rows // _BM + docs + 1
     n_kv = rows // _BKV + docs + 1
-    words = _SCHED_HDR + 4 * (n_q + n_kv) + 5 * docs + 2
-    n_tt = -(-max(1, max_doc_len if not fixed else tokens) // _BT)
-    return (4 * words + 255) & ~255, heads * (n_tt + 1) * rows
+    words = _SCHED_HDR + _TILE_WORDS * (n_q + n_kv) + 6 * docs + 2
+    if fixed:
+        entries = batch * table_entries(tokens)
+    elif lengths is not None:
+        entries = max(1, sum(table_entries(int(n)) for n in lengths))
+    else:
+        entries = table_entries_bound(tokens, max_doc_len)
+    return (4 * words + 255) & ~255, heads * entries
+
+
+# cu_seqlens tensors already copied to the host: (weak reference, version, tuple of values), newest last
+_host_cu_cache = []
+_HOST_CU_CACHE_SIZE = 8
+
+
+def _version_of(t):
+    """The in-place modification counter of a tensor, or None where PyTorch keeps none (tensors
+    created under ``torch.inference_mode()`` raise on ``_version``)."""
+    try:
+        return t._version
+    except RuntimeError:
+        return None
+
+
+def host_cu_seqlens(cu_seqlens: torch.Tensor, allow_sync: bool = True) -> Optional[Tuple[int, ...]]:
+    """The values of a cu_seqlens tensor on the host, remembered per tensor object for as long as it
+    comes back unmodified; None when they are not known and may not be fetched (``allow_sync``
+    False, SBA_SYNC_FREE, torch.compile).  A write through ``cu_seqlens.data`` does not advance the
+    tensor's version counter and is therefore not seen: do not rewrite a cu_seqlens tensor that
+    way between calls."""
+    if torch.compiler.is_compiling():
+        return None
+    version = _version_of(cu_seqlens)
+    if version is not None:
+        for i in range(len(_host_cu_cache) - 1, -1, -1):
+            ref, ver, vals = _host_cu_cache[i]
+            if ref() is cu_seqlens:
+                if ver == version:
+                    return vals
+                del _host_cu_cache[i]
+                break
+    if cu_seqlens.is_cuda and (not allow_sync or SYNC_FREE):
+        return None
+    vals = tuple(int(x) for x in cu_seqlens.tolist())   # the one synchronisation per tensor
+    if version is not None:
+        _host_cu_cache[:] = [e for e in _host_cu_cache if e[0]() is not None][-(_HOST_CU_CACHE_SIZE - 1):]
+        _host_cu_cache.append((weakref.ref(cu_seqlens), version, vals))
+    return vals
+
+
+def remember_host_cu(cu_seqlens: torch.Tensor, vals: Sequence[int]) -> None:
+    """Associate host values with a tensor whose contents are already known (the view without the
+    leading zero that ``sb_attn_varlen`` passes on)."""
+    version = _version_of(cu_seqlens)
+    if version is None or torch.compiler.is_compiling():
+        return
+    _host_cu_cache[:] = [e for e in _host_cu_cache if e[0]() is not None][-(_HOST_CU_CACHE_SIZE - 1):]
+    _host_cu_cache.append((weakref.ref(cu_seqlens), version, tuple(int(x) for x in vals)))
+
+
+def _doc_lengths(cu_vals: Sequence[int], tokens: int) -> Tuple[int, ...]:
+    """Document lengths from inclusive cumulative ends (no leading zero); raises on what the device
+    scheduler would flag as SBA_STATUS_BAD_CU."""
+    prev, out = 0, []
+    for end in cu_vals:
+        if end < prev or end > tokens:
+            raise ValueError("sb_attn_varlen: " + nat.STATUS_MESSAGES[1])
+        out.append(end - prev)
+        prev = end
+    return tuple(out)
 
 
 _warned_dtypes = set()
@@ -117,25 +209,27 @@ def _ptr(t: Optional[torch.Tensor]):
 # ---------------------------------------------------------------------------------------------
 # launchers: everything is allocated by the caller
 # ---------------------------------------------------------------------------------------------
+def _nbytes(t: Optional[torch.Tensor]) -> int:
+    return 0 if t is None else t.numel() * t.element_size()
+
+
 def _launch_fwd(fixed: bool, q, k, v, cu_seqlens, max_doc_len: int, logit_scale: float, attend_current: bool,
                 product: bool, fused: bool, o, rem, table, sched, weights=None) -> None:
     nat.require_gpu(q)
     lib = nat.load()
     q, k, v = _aligned(q), _aligned(k), _aligned(v)
     prob, _keep = _problem(q, fixed, cu_seqlens, max_doc_len, logit_scale, attend_current, product, fused)
-    need, _ = workspace_sizes(fixed, prob.batch, prob.heads, prob.tokens, prob.n_docs, prob.max_doc_len)
-    if sched.numel() * sched.element_size() < need:
-        raise ValueError("schedule workspace too small")
     name = ("sba_attn_fwd" if fixed else "sba_varlen_fwd") + ("_weights" if weights is not None else "")
     fn = getattr(lib, name)
-    extra = () if weights is None else (weights.data_ptr(),)
+    extra = () if weights is None else (weights.data_ptr(), _nbytes(weights))
     with torch.cuda.device(q.device):
         stream = nat.stream_ptr(q.device)
-        nat.check(lib.sba_build_schedule(ctypes.byref(prob), sched.data_ptr(), stream), "sba_build_schedule")
-        code = fn(ctypes.byref(prob), sched.data_ptr(),
+        # every workspace goes in with its size: the library answers SBA_E_WORKSPACE instead of overrunning one
+        nat.check(lib.sba_build_schedule(ctypes.byref(prob), sched.data_ptr(), _nbytes(sched), stream), "sba_build_schedule")
+        code = fn(ctypes.byref(prob), sched.data_ptr(), _nbytes(sched),
                   ctypes.byref(nat.view4(q, fixed)), ctypes.byref(nat.view4(k, fixed)),
                   ctypes.byref(nat.view4(v, fixed)), ctypes.byref(nat.view4(o, fixed)),
-                  ctypes.byref(nat.view4(rem, fixed, per_row=True)), _ptr(table), *extra, stream)
+                  ctypes.byref(nat.view4(rem, fixed, per_row=True)), _ptr(table), _nbytes(table), *extra, stream)
     nat.check(code, name)
 
 
@@ -147,12 +241,14 @@ def _launch_bwd(fixed: bool, do, dr, q, k, v, cu_seqlens, max_doc_len: int, logi
     prob, _keep = _problem(q, fixed, cu_seqlens, max_doc_len, logit_scale, attend_current, product, fused)
     fn = lib.sba_attn_bwd if fixed else lib.sba_varlen_bwd
     drv = dr if dr is not None and dr.numel() else None
+    if table.numel() == 0:
+        raise ValueError("the backward needs the carry table of a forward that ran with gradients enabled")
     with torch.cuda.device(q.device):
-        code = fn(ctypes.byref(prob), sched.data_ptr(),
+        code = fn(ctypes.byref(prob), sched.data_ptr(), _nbytes(sched),
                   ctypes.byref(nat.view4(q, fixed)), ctypes.byref(nat.view4(k, fixed)),
                   ctypes.byref(nat.view4(v, fixed)), ctypes.byref(nat.view4(do, fixed)),
                   ctypes.byref(nat.view4(drv, fixed, per_row=True)),
-                  table.data_ptr(), gtab.data_ptr(),
+                  table.data_ptr(), gtab.data_ptr(), min(_nbytes(table), _nbytes(gtab)),
                   ctypes.byref(nat.view4(dq, fixed)), ctypes.byref(nat.view4(dk, fixed)),
                   ctypes.byref(nat.view4(dv, fixed)), nat.stream_ptr(q.device))
     nat.check(code, "sba_attn_bwd" if fixed else "sba_varlen_bwd")
@@ -218,6 +314,7 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
     dpad = _padded_dim(d)
     product = PRODUCT_SPACE
     qp, kp, vp = (_prep(t, dpad) for t in (q, k, v))
+    lengths = None
     if fixed:
         B, H, T, _ = qp.shape
         n_docs, max_len, cu = 0, T, None
@@ -227,7 +324,13 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
         cu = _check_cu(cu_seqlens, q)
         n_docs = cu.numel()
         max_len = T if max_seqlens is None else max(1, min(int(max_seqlens), T))
-    sched_bytes, table_floats = workspace_sizes(fixed, B, H, T, n_docs, max_len)
+        cu_vals = host_cu_seqlens(cu)
+        if cu_vals is not None:
+            # lengths known on the host: malformed input raises here, the tables get their exact
+            # size, and results do not depend on max_seqlens at all
+            lengths = _doc_lengths(cu_vals, T)
+            max_len = max(1, max(lengths, default=1))
+    sched_bytes, table_floats = workspace_sizes(fixed, B, H, T, n_docs, max_len, lengths)
     # Every row is written by the library: rows of documents by the forward kernel, rows that
     # belong to no document are cleared (upstream leaves those uninitialised).
     o = torch.empty_like(qp)
@@ -245,7 +348,7 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
         _compileable_forward(qp, kp, vp, cu, max_len, float(inv_temp), bool(attend_current), product,
                              bool(fused), o, rem, table, sched)
         if VALIDATE and not torch.compiler.is_compiling():
-            check_status(sched)
+            check_status(sched, table, H)
     if dpad != d or q.dtype != torch.bfloat16:
         o = o[..., :d].to(q.dtype)
         rem = rem.to(q.dtype)
@@ -253,11 +356,38 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
     return (o, rem, state, weights) if return_attention else (o, rem, state)
 
 
-def check_status(sched: torch.Tensor) -> None:
-    """Read the scheduler's status word back (synchronises) and raise on malformed input."""
-    status = int(sched[:4].view(torch.int32).item())
+def check_status(sched: torch.Tensor, table: Optional[torch.Tensor] = None, heads: int = 1) -> None:
+    """Read the scheduler's status words back (synchronises) and raise on malformed cu_seqlens or on
+    carry tables smaller than the documents need."""
+    hdr = sched[:16].view(torch.int32).tolist()
+    status, need = hdr[0], hdr[3]
+    if status == 0 and table is not None and table.numel() and need > table.numel() // heads:
+        status = 4
     if status != 0:
         raise ValueError("sb_attn_varlen: " + nat.STATUS_MESSAGES.get(status, f"scheduler status {status}"))
+
+
+# One gradient table per (device, stream, size), reused by every backward of that shape: the dk/dv
+# pass of one backward has read it before the dq pass of the next (same stream) writes it.
+_gtab_cache = {}
+
+
+def _grad_table(like: torch.Tensor) -> torch.Tensor:
+    if torch.compiler.is_compiling():
+        return torch.empty_like(like)
+    key = (like.device, torch.cuda.current_stream(like.device).cuda_stream, like.numel())
+    t = _gtab_cache.get(key)
+    if t is None:
+        if len(_gtab_cache) >= 4:
+            _gtab_cache.clear()
+        t = _gtab_cache[key] = torch.empty_like(like)
+    return t
+
+
+def release_workspaces() -> None:
+    """Drop the cached gradient tables and host copies of cu_seqlens."""
+    _gtab_cache.clear()
+    del _host_cu_cache[:]
 
 
 def run_backward(q, k, v, do, drem, fixed: bool, state, inv_temp: float, attend_current: bool, dkdv_dtype=None,
@@ -275,7 +405,7 @@ def run_backward(q, k, v, do, drem, fixed: bool, state, inv_temp: float, attend_
         if torch.compiler.is_compiling():
             dremp = dremp.contiguous()
     dq, dk, dv = torch.empty_like(qp), torch.empty_like(kp), torch.empty_like(vp)
-    gtab = torch.empty_like(table)
+    gtab = _grad_table(table)
     if fixed:
         _compileable_bwd(dop, dremp, qp, kp, vp, float(inv_temp), bool(attend_current), product, bool(fused),
                          table, sched, gtab, dq, dk, dv)

@@ -5,7 +5,6 @@ argument order, defaults and return values (``sb_attn_varlen`` :71-78, ``sb_attn
 :81-82, ``StickBreakingAttention`` :24-68).  The device work is done by libsba.so.
 """
 import math
-import weakref
 
 import torch
 
@@ -32,40 +31,30 @@ def varlen_bwd(do, dr, q, k, v, state, logit_scale, attend_current=False, fused=
     return _ops.run_backward(q, k, v, do, dr, False, state, logit_scale, attend_current, fused=fused)
 
 
-# The last cu_seqlens tensor whose first entry was read back and found to be zero.
-_zero_start_checked = None
-
-
-def _version_of(t):
-    """The in-place modification counter of a tensor, or None where PyTorch keeps none (tensors
-    created under ``torch.inference_mode()`` raise on ``_version``)."""
-    try:
-        return t._version
-    except RuntimeError:
-        return None
-
-
 def _starts_at_zero(cu_seqlens) -> bool:
     """``cu_seqlens[0] == 0``, upstream's check (sb_varlen/__init__.py:73).  Reading one element of a
     device tensor stalls the host until the GPU has drained, and a model passes the same
-    cu_seqlens to every layer, so the answer is remembered for as long as the same tensor object
-    comes back unmodified: one synchronisation per batch instead of one per call.  Tensors without
-    a modification counter (inference tensors) are checked on every call.  A write through
-    ``cu_seqlens.data`` does not advance the counter and is therefore not seen: do not rewrite a
-    cu_seqlens tensor that way between calls."""
-    global _zero_start_checked
+    cu_seqlens to every layer, so the whole tensor is copied to the host once per tensor object and
+    version (``_ops.host_cu_seqlens``, which the launcher uses as well): one synchronisation per
+    batch instead of one per call.  Tensors without a modification counter (inference tensors) are
+    read on every call."""
     if torch.compiler.is_compiling():
         return bool(cu_seqlens[0] == 0)
-    version = _version_of(cu_seqlens)
-    if version is None:
+    vals = _ops.host_cu_seqlens(cu_seqlens)
+    if vals is None:                      # SBA_SYNC_FREE: upstream's assertion still needs this one value
         return bool(cu_seqlens[0] == 0)
-    seen = _zero_start_checked
-    if seen is not None and seen[0]() is cu_seqlens and seen[1] == version:
-        return True
-    ok = bool(cu_seqlens[0] == 0)
-    if ok:
-        _zero_start_checked = (weakref.ref(cu_seqlens), version)
-    return ok
+    return len(vals) > 0 and vals[0] == 0
+
+
+def _strip_leading_zero(cu_seqlens):
+    """``cu_seqlens[1:]`` (upstream sb_varlen/__init__.py:74), carrying the host copy of the values
+    over to the new view so that the launcher does not read them back again."""
+    stripped = cu_seqlens[1:]
+    if not torch.compiler.is_compiling():
+        vals = _ops.host_cu_seqlens(cu_seqlens, allow_sync=False)
+        if vals is not None:
+            _ops.remember_host_cu(stripped, vals[1:])
+    return stripped
 
 
 class StickBreakingAttention(torch.autograd.Function):
@@ -97,7 +86,7 @@ def sb_attn_varlen(q, k, v, cu_seqlens, max_seqlens=None, inv_temp=None, zero_st
     rem [heads, total_tokens])."""
     if zero_start:
         assert _starts_at_zero(cu_seqlens)
-        cu_seqlens = cu_seqlens[1:]
+        cu_seqlens = _strip_leading_zero(cu_seqlens)
     if inv_temp is None:
         inv_temp = 1 / math.sqrt(q.size(-1))
     return sb_attn_varlen_(q, k, v, inv_temp, cu_seqlens, max_seqlens, attend_current)
@@ -138,7 +127,7 @@ def sb_attn_varlen_fused(q, k, v, cu_seqlens, max_seqlens=None, inv_temp=None, z
     the extra passes over ``o`` and ``v`` in forward and backward."""
     if zero_start:
         assert _starts_at_zero(cu_seqlens)
-        cu_seqlens = cu_seqlens[1:]
+        cu_seqlens = _strip_leading_zero(cu_seqlens)
     if inv_temp is None:
         inv_temp = 1 / math.sqrt(q.size(-1))
     return StickBreakingAttentionFused.apply(q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current)

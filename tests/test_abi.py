@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for s in syms:
         assert hasattr(lib, s), f"{s} declared in include/sba.h but not exported"
     assert sorted(nat.EXPORTS) == syms
-    assert lib.sba_version() == 101
+    assert lib.sba_version() == 200
 
 
 def problem(**kw):
@@ -35,17 +35,62 @@ def problem(**kw):
     return nat.SbaProblem(*[base[f[0]] for f in nat.SbaProblem._fields_])
 
 
+def _entries(L):
+    nb = -(-L // 32)
+    return sum(L - 32 * b for b in range(nb)) + L      # rows at or below each 32-key block, plus one per row
+
+
 def test_workspace_sizes():
     lib = nat.load()
     p = problem()
     sched = lib.sba_schedule_bytes(ctypes.byref(p))
-    # two tile lists (16 B per tile): query tiles and key tiles, each bounded by tokens/128 + docs
-    assert 16 * (128 + 8 + 128 + 8) <= sched <= 16 * (128 + 128 + 32) + 1024
-    # one plane per 32-key block of the longest document plus one plane of per-row values
-    assert lib.sba_table_bytes(ctypes.byref(p)) == 32 * (128 + 1) * 16384 * 4
+    # two tile lists (32 B per tile): query tiles and key tiles, each bounded by tokens/128 + docs
+    assert 32 * (128 + 8 + 128 + 8) <= sched <= 32 * (128 + 128 + 32) + 1024
+    # no lengths: four documents of max_doc_len = 4096 tokens are the worst split of 16384 tokens
+    assert lib.sba_table_bytes(ctypes.byref(p)) == 32 * 4 * _entries(4096) * 4
+    # exact, from host lengths (the headline workload's documents): under 100 MiB
+    lengths = [4026, 2261, 1563, 566, 1189, 615, 3465, 2699]
+    arr = (ctypes.c_int64 * len(lengths))(*lengths)
+    exact = lib.sba_table_bytes_for_lengths(ctypes.byref(p), arr, len(lengths))
+    assert exact == 32 * sum(_entries(n) for n in lengths) * 4
+    assert exact < 100 * 2 ** 20 < lib.sba_table_bytes(ctypes.byref(p))
+    # a length beyond the token count is refused
+    bad = (ctypes.c_int64 * 1)(20000)
+    assert lib.sba_table_bytes_for_lengths(ctypes.byref(p), bad, 1) == 0
     pf = problem(batch=4, heads=16, tokens=2048, n_docs=0, max_doc_len=2048, head_dim=64,
                  flags=nat.FLAG_FIXED_LENGTH, cu_seqlens=None)
-    assert lib.sba_table_bytes(ctypes.byref(pf)) == 16 * (64 + 1) * 4 * 2048 * 4
+    assert lib.sba_table_bytes(ctypes.byref(pf)) == 16 * 4 * _entries(2048) * 4
+
+
+def test_undersized_workspaces_are_refused_on_the_host():
+    """Every workspace travels with its size; what the host can check comes back as SBA_E_WORKSPACE
+    (-6) before anything is launched (no GPU is touched: argument checks come first)."""
+    lib = nat.load()
+    p = problem()
+    need = lib.sba_schedule_bytes(ctypes.byref(p))
+    v = nat.SbaView(0x1000, 0, 128 * 16384, 128)
+    r = nat.SbaView(0x1000, 0, 16384, 1)
+    vs = [ctypes.byref(x) for x in (v, v, v, v, r)]
+    sched = ctypes.c_void_p(0x1000)
+    assert lib.sba_build_schedule(ctypes.byref(p), sched, need - 1, None) == -6
+    assert lib.sba_varlen_fwd(ctypes.byref(p), sched, need - 1, *vs, None, 0, None) == -6
+    assert lib.sba_varlen_fwd(ctypes.byref(p), sched, need, *vs, ctypes.c_void_p(0x1000), 0, None) in (-6, -7)
+    assert lib.sba_varlen_fwd_weights(ctypes.byref(p), sched, need, *vs, None, 0, ctypes.c_void_p(0x1000), 1024, None) == -6
+    bw = [ctypes.byref(x) for x in (v, v, v, v, r)]
+    outs = [ctypes.byref(v)] * 3
+    assert lib.sba_varlen_bwd(ctypes.byref(p), sched, need - 1, *bw, ctypes.c_void_p(0x1000),
+                              ctypes.c_void_p(0x1000), 1 << 30, *outs, None) == -6
+    # fixed-length: the table need is known on the host
+    pf = problem(batch=4, heads=16, tokens=2048, n_docs=0, max_doc_len=2048, head_dim=64,
+                 flags=nat.FLAG_FIXED_LENGTH, cu_seqlens=None)
+    needf = lib.sba_schedule_bytes(ctypes.byref(pf))
+    tbl = lib.sba_table_bytes(ctypes.byref(pf))
+    vf = nat.SbaView(0x1000, 16 * 2048 * 64, 2048 * 64, 64)
+    rf = nat.SbaView(0x1000, 16 * 2048, 2048, 1)
+    vsf = [ctypes.byref(x) for x in (vf, vf, vf, vf, rf)]
+    assert lib.sba_attn_fwd(ctypes.byref(pf), sched, needf, *vsf, ctypes.c_void_p(0x1000), tbl - 4, None) == -6
+    assert lib.sba_attn_bwd(ctypes.byref(pf), sched, needf, *vsf, ctypes.c_void_p(0x1000), ctypes.c_void_p(0x1000),
+                            tbl - 4, *[ctypes.byref(vf)] * 3, None) == -6
 
 
 @pytest.mark.parametrize("kw,code", [
@@ -56,11 +101,11 @@ def test_bad_problems_are_rejected_on_the_host(kw, code):
     lib = nat.load()
     p = problem(**kw)
     assert lib.sba_schedule_bytes(ctypes.byref(p)) == 0
-    assert lib.sba_build_schedule(ctypes.byref(p), ctypes.c_void_p(0x1000), None) == code
+    assert lib.sba_build_schedule(ctypes.byref(p), ctypes.c_void_p(0x1000), 1 << 20, None) == code
     v = nat.SbaView(0x1000, 0, 128 * 16384, 128)
     r = nat.SbaView(0x1000, 0, 16384, 1)
-    assert lib.sba_varlen_fwd(ctypes.byref(p), ctypes.c_void_p(0x1000), ctypes.byref(v), ctypes.byref(v),
-                              ctypes.byref(v), ctypes.byref(v), ctypes.byref(r), None, None) == code
+    assert lib.sba_varlen_fwd(ctypes.byref(p), ctypes.c_void_p(0x1000), 1 << 20, ctypes.byref(v), ctypes.byref(v),
+                              ctypes.byref(v), ctypes.byref(v), ctypes.byref(r), None, 0, None) == code
 
 
 def test_misaligned_stride_and_null_views_are_rejected():
@@ -70,8 +115,8 @@ def test_misaligned_stride_and_null_views_are_rejected():
     bad = nat.SbaView(0x1000, 0, 128 * 16384 + 2, 128)
     null = nat.SbaView(None, 0, 0, 0)
     r = nat.SbaView(0x1000, 0, 16384, 1)
-    args = lambda q: (ctypes.byref(p), ctypes.c_void_p(0x1000), ctypes.byref(q), ctypes.byref(good),
-                      ctypes.byref(good), ctypes.byref(good), ctypes.byref(r), None, None)
+    args = lambda q: (ctypes.byref(p), ctypes.c_void_p(0x1000), 1 << 20, ctypes.byref(q), ctypes.byref(good),
+                      ctypes.byref(good), ctypes.byref(good), ctypes.byref(r), None, 0, None)
     assert lib.sba_varlen_fwd(*args(bad)) == -5
     assert lib.sba_varlen_fwd(*args(null)) == -1
     assert b"16-byte" in lib.sba_error_string(-5)
@@ -124,30 +169,54 @@ def test_operators_are_registered_under_the_upstream_names():
         assert hasattr(torch.ops.stickbreaking_attention, name)
 
 
-def test_leading_zero_check_is_cached_per_tensor_object():
-    """Host logic only: the answer for one cu_seqlens tensor is reused until the tensor is modified
-    in place or another tensor arrives (upstream asserts on every call, sb_varlen/__init__.py:73)."""
+def test_host_copy_of_cu_seqlens_is_cached_per_tensor_object():
+    """Host logic only: the values of one cu_seqlens tensor are fetched once and reused until the
+    tensor is modified in place or another tensor arrives (upstream reads cu_seqlens[0] back on every
+    call for its assertion, sb_varlen/__init__.py:73)."""
     import torch
-    from stickbreaking_attention import sb_varlen
+    from stickbreaking_attention import _ops, sb_varlen
+    _ops.release_workspaces()
     cu = torch.tensor([0, 5, 9], dtype=torch.int32)
     assert sb_varlen._starts_at_zero(cu)
-    assert sb_varlen._zero_start_checked[0]() is cu
+    assert _ops._host_cu_cache[-1][0]() is cu and _ops._host_cu_cache[-1][2] == (0, 5, 9)
+    n = len(_ops._host_cu_cache)
+    assert sb_varlen._starts_at_zero(cu) and len(_ops._host_cu_cache) == n       # served from the cache
+    stripped = sb_varlen._strip_leading_zero(cu)
+    assert _ops.host_cu_seqlens(stripped, allow_sync=False) == (5, 9)              # carried over to the view
     same_values = torch.tensor([0, 5, 9], dtype=torch.int32)
-    assert sb_varlen._starts_at_zero(same_values) and sb_varlen._zero_start_checked[0]() is same_values
-    same_values[0] = 2
+    assert sb_varlen._starts_at_zero(same_values) and _ops._host_cu_cache[-1][0]() is same_values
+    same_values[0] = 2                                                             # in-place write: new version
     assert not sb_varlen._starts_at_zero(same_values)
+    assert _ops.host_cu_seqlens(same_values) == (2, 5, 9)
     assert not sb_varlen._starts_at_zero(torch.tensor([1, 4]))
+    with pytest.raises(ValueError):
+        _ops._doc_lengths((5, 3), 10)          # not monotone
+    with pytest.raises(ValueError):
+        _ops._doc_lengths((5, 12), 10)         # beyond the token count
+    assert _ops._doc_lengths((5, 5, 9), 10) == (5, 0, 4)
 
 
 def test_leading_zero_check_works_on_inference_tensors():
-    """Tensors created under torch.inference_mode() have no version counter: the check must fall
-    back to reading the first element every time instead of raising."""
+    """Tensors created under torch.inference_mode() have no version counter: the check must read
+    the values every time instead of raising."""
     import torch
-    from stickbreaking_attention import sb_varlen
+    from stickbreaking_attention import _ops, sb_varlen
+    _ops.release_workspaces()
     with torch.inference_mode():
         cu = torch.tensor([0, 5, 9], dtype=torch.int32)
         bad = torch.tensor([3, 5, 9], dtype=torch.int32)
         assert sb_varlen._starts_at_zero(cu) and sb_varlen._starts_at_zero(cu)
         assert not sb_varlen._starts_at_zero(bad)
     assert sb_varlen._starts_at_zero(cu)          # also outside the mode, on the inference tensor
-    assert sb_varlen._zero_start_checked is None or sb_varlen._zero_start_checked[0]() is not cu
+    assert all(e[0]() is not cu for e in _ops._host_cu_cache)
+
+
+def test_python_table_formula_with_lengths_matches_the_library():
+    from stickbreaking_attention import _ops
+    lib = nat.load()
+    p = problem()
+    lengths = [4026, 2261, 1563, 566, 1189, 615, 3465, 2699, 0, 1, 33]
+    p.tokens = sum(lengths)
+    arr = (ctypes.c_int64 * len(lengths))(*lengths)
+    _, table = _ops.workspace_sizes(False, 1, p.heads, p.tokens, len(lengths), 0, lengths)
+    assert 4 * table == lib.sba_table_bytes_for_lengths(ctypes.byref(p), arr, len(lengths))

@@ -110,14 +110,46 @@ def _poison_free_blocks(shape, n=6):
     del blocks
 
 
-def test_rejected_cu_seqlens_give_zero_outputs():
-    from stickbreaking_attention import sb_attn_varlen
+def test_rejected_cu_seqlens_raise_or_poison_the_outputs(monkeypatch):
+    """Malformed cu_seqlens: with the host copy of cu_seqlens (the default) the call raises before
+    anything is launched; without it (SBA_SYNC_FREE, torch.compile) the device scheduler refuses
+    the input, no attention is computed and every output element is NaN -- never a plausible value."""
+    from stickbreaking_attention import _ops, sb_attn_varlen
     q = torch.randn(2, 256, 64, device=DEV).to(torch.bfloat16)
+    bad = torch.tensor([100, 50, 256], dtype=torch.int32, device=DEV)
+    with pytest.raises(ValueError, match="non-decreasing"):
+        sb_attn_varlen(q, q, q, bad, 256, zero_start=False)
+    monkeypatch.setattr(_ops, "SYNC_FREE", True)
+    _ops.release_workspaces()
     _poison_free_blocks((2, 256, 64))
-    with torch.no_grad():
-        o, rem = sb_attn_varlen(q, q, q, torch.tensor([100, 50, 256], dtype=torch.int32, device=DEV), 256, zero_start=False)
+    qg = q.clone().requires_grad_()
+    o, rem = sb_attn_varlen(qg, qg, qg, bad, 256, zero_start=False)
+    (dq,) = torch.autograd.grad(o, (qg,), torch.ones_like(o))
     torch.cuda.synchronize()
-    assert (o == 0).all() and (rem == 0).all()
+    assert torch.isnan(o).all() and torch.isnan(rem).all() and torch.isnan(dq).all()
+
+
+def test_understated_max_seqlens(monkeypatch):
+    """Upstream silently drops rows when max_seqlens under-states a document (sb_varlen_fwd.py:478).
+    Here results do not depend on max_seqlens when the lengths are known on the host; without them
+    the tables sized from the understated bound are too small, which the device detects: NaN
+    outputs, and a ValueError when validation is switched on."""
+    from stickbreaking_attention import _ops, sb_attn_varlen
+    lengths = [700, 300]
+    q, k, v, do = orc.make_inputs((2, 1000, 64), 77)
+    ref = oracle_varlen(q, k, v, do, lengths)
+    got = run_varlen(q, k, v, do, lengths, max_seqlens=64)          # default: lengths read back once, exact tables
+    check_all(got, ref)
+    monkeypatch.setattr(_ops, "SYNC_FREE", True)
+    _ops.release_workspaces()
+    got = run_varlen(q, k, v, do, lengths, max_seqlens=64)
+    for t in got:
+        assert torch.isnan(t).all()
+    got = run_varlen(q, k, v, do, lengths, max_seqlens=700)         # a correct bound: same results as above
+    check_all(got, ref)
+    monkeypatch.setattr(_ops, "VALIDATE", True)
+    with pytest.raises(ValueError, match="too small"):
+        run_varlen(q, k, v, do, lengths, max_seqlens=64)
 
 
 def test_no_documents_give_zero_outputs():
@@ -356,16 +388,17 @@ def test_other_dtypes_are_computed_in_bf16(dtype):
 
 def test_malformed_cu_seqlens_are_reported(monkeypatch):
     from stickbreaking_attention import _ops, sb_attn_varlen
-    monkeypatch.setattr(_ops, "VALIDATE", True)
     q = torch.zeros(2, 256, 64, dtype=torch.bfloat16, device=DEV)
-    with pytest.raises(ValueError, match="non-decreasing"):
-        sb_attn_varlen(q, q, q, torch.tensor([100, 50, 256], dtype=torch.int32, device=DEV), 256, zero_start=False)
-    with pytest.raises(ValueError, match="non-decreasing"):
-        sb_attn_varlen(q, q, q, torch.tensor([100, 300], dtype=torch.int32, device=DEV), 256, zero_start=False)
-    with pytest.raises(ValueError, match="longer than max_seqlens"):
-        sb_attn_varlen(q, q, q, torch.tensor([200, 256], dtype=torch.int32, device=DEV), 64, zero_start=False)
-    with pytest.raises(AssertionError):
-        sb_attn_varlen(q, q, q, torch.tensor([5, 256], dtype=torch.int32, device=DEV), 256, zero_start=True)
+    for sync_free in (False, True):          # host-side check by default, device status word otherwise
+        monkeypatch.setattr(_ops, "SYNC_FREE", sync_free)
+        monkeypatch.setattr(_ops, "VALIDATE", sync_free)
+        _ops.release_workspaces()
+        with pytest.raises(ValueError, match="non-decreasing"):
+            sb_attn_varlen(q, q, q, torch.tensor([100, 50, 256], dtype=torch.int32, device=DEV), 256, zero_start=False)
+        with pytest.raises(ValueError, match="non-decreasing"):
+            sb_attn_varlen(q, q, q, torch.tensor([100, 300], dtype=torch.int32, device=DEV), 256, zero_start=False)
+        with pytest.raises(AssertionError):
+            sb_attn_varlen(q, q, q, torch.tensor([5, 256], dtype=torch.int32, device=DEV), 256, zero_start=True)
     torch.cuda.synchronize()
 
 
@@ -420,17 +453,24 @@ def test_torch_compile_traces_through_the_registered_operators():
         assert torch.equal(a, b)
 
 
-def test_zero_start_check_is_remembered_per_tensor():
-    """The leading-zero assertion reads the device once per cu_seqlens tensor, not once per call, and
-    still fires for a new or modified tensor."""
-    from stickbreaking_attention import sb_attn_varlen
-    from stickbreaking_attention import sb_varlen
+def test_cu_seqlens_are_read_back_once_per_tensor():
+    """The leading-zero assertion and the table sizing read the device once per cu_seqlens tensor,
+    not once per call, and still see a new or modified tensor."""
+    from stickbreaking_attention import _ops, sb_attn_varlen
+    _ops.release_workspaces()
     q = torch.zeros(2, 256, 64, dtype=torch.bfloat16, device=DEV)
     cu = torch.tensor([0, 100, 256], dtype=torch.int32, device=DEV)
     sb_attn_varlen(q, q, q, cu, 256)
-    assert sb_varlen._zero_start_checked[0]() is cu
-    sb_attn_varlen(q, q, q, cu, 256)                       # same tensor: no second read
-    cu[0] = 3                                              # in-place change bumps the version: checked again
+    assert any(e[0]() is cu and e[2] == (0, 100, 256) for e in _ops._host_cu_cache)
+    reads = []
+    orig = torch.Tensor.tolist
+    try:
+        torch.Tensor.tolist = lambda self: (reads.append(1), orig(self))[1]
+        sb_attn_varlen(q, q, q, cu, 256)                   # same tensor: no second read
+        assert not reads
+    finally:
+        torch.Tensor.tolist = orig
+    cu[0] = 3                                              # in-place change bumps the version: read again
     with pytest.raises(AssertionError):
         sb_attn_varlen(q, q, q, cu, 256)
     with pytest.raises(AssertionError):

@@ -38,8 +38,8 @@ def _forward_pair(lengths, H, d, seed):
     before = torch.cuda.memory_allocated(dev)
     nat.check(lib.sba_varlen_fwd_static(ctypes.byref(prob), *views(o_a, rem_a), stream), "sba_varlen_fwd_static")
     assert torch.cuda.memory_allocated(dev) == before
-    nat.check(lib.sba_build_schedule(ctypes.byref(prob), sched.data_ptr(), stream), "sba_build_schedule")
-    nat.check(lib.sba_varlen_fwd(ctypes.byref(prob), sched.data_ptr(), *views(o_b, rem_b), None, stream), "sba_varlen_fwd")
+    nat.check(lib.sba_build_schedule(ctypes.byref(prob), sched.data_ptr(), sched.numel(), stream), "sba_build_schedule")
+    nat.check(lib.sba_varlen_fwd(ctypes.byref(prob), sched.data_ptr(), sched.numel(), *views(o_b, rem_b), None, 0, stream), "sba_varlen_fwd")
     torch.cuda.synchronize()
     return (q, k, v), (o_a, rem_a), (o_b, rem_b)
 
