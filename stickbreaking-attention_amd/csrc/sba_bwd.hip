@@ -108,6 +108,7 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   // double-buffered, filled by asynchronous global -> LDS copies.
   __shared__ __attribute__((aligned(16))) unsigned short Ks[2 * TILE];
   __shared__ __attribute__((aligned(16))) unsigned short Vs[2 * TILE];
+  __shared__ float Cst[NT / 64][32];   // per wave: a table value waiting for the next tile's top
 
   // Header words and this workgroup's tile are fetched together (the grid never exceeds the
   // allocated list, so the tile read is safe before the count is known): one round trip.
@@ -194,22 +195,24 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
       toff[u][db] = swz_off<D>(r, col >> 3) + (col & 7);
     }
   }
-  const int64_t tab0 = (int64_t)head * a.tab_stride + t.tab_base + qrow;   // this row's entries of the document's table area
+  // the document's area of the two tables (uniform); a lane adds its row and a block's 32-bit offset
+  const int64_t tab0 = (int64_t)head * a.tab_stride + t.tab_base;
   const float* stick = a.stick + tab0;
   float* gtab = a.gtab + tab0;
   // the dk/dv pass takes d(rem) from the last plane of the gradient table
-  if (qvalid && h == 0) gtab[tab_rowplane(t.doc_len)] = dr;
+  if (qvalid && h == 0) gtab[(unsigned)(tab_rowplane32(t.doc_len) + qrow)] = dr;
 
   // stick carries of the two sub-blocks of a tile (neutral where the sub-block is skipped)
   auto carries = [&](int kt, float (&ce)[2]) {
 #pragma unroll
     for (int sb = 0; sb < 2; ++sb) {
       ce[sb] = PROD ? 1.0f : 0.0f;
-      if (qvalid && kt <= kt_last && !sub_skip<AC>(kt * BN + 32 * sb, qw0)) ce[sb] = stick[tab_seg(t.doc_len, 2 * kt + sb)];
+      if (qvalid && kt <= kt_last && !sub_skip<AC>(kt * BN + 32 * sb, qw0)) ce[sb] = stick[(unsigned)(tab_seg32(t.doc_len, 2 * kt + sb) + qrow)];
     }
   };
   float ce[2], ce_next[2];
   carries(0, ce);
+  int pend_ix = -1;         // table entry of a prefix that is still to be stored (same for the whole wave)
 
   // One tile step; the buffer index is a compile-time constant so that every LDS address is a
   // fixed register plus an immediate.
@@ -218,6 +221,14 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
     // tile kt has landed and every wave is done with the tile before it
     wait_loads<0>();
     lds_barrier();
+    // Table stores only ever go out here, at the top of a tile: the vmcnt wait above also waits
+    // for the acknowledgement of stores (well over a thousand cycles), so a store issued in the
+    // middle of a tile would stall the top of the next one.  The prefix of the second sub-block
+    // therefore waits in LDS (no register to spare) until the next tile begins.
+    if (pend_ix >= 0) {
+      if (qvalid && h == 0) gtab[(unsigned)(pend_ix + qrow)] = Cst[w][n];
+      pend_ix = -1;
+    }
     // the next tile's carries go out before its tile copy; neither is waited for in this step
     carries(kt + 1, ce_next);
     if (kt < kt_last) {
@@ -230,8 +241,13 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
     for (int sb = 0; sb < 2; ++sb) {
       const int k0 = kt * BN + 32 * sb;
       if (sub_skip<AC>(k0, qw0)) continue;
-      const int64_t tix = tab_seg(t.doc_len, 2 * kt + sb);
-      if (qvalid && h == 0) gtab[tix] = carry_c;
+      const int tix = tab_seg32(t.doc_len, 2 * kt + sb);   // (uniform)
+      if (sb == 0) {
+        if (qvalid && h == 0) gtab[(unsigned)(tix + qrow)] = carry_c;
+      } else {
+        pend_ix = tix;
+        if (h == 0) Cst[w][n] = carry_c;
+      }
       // LDS latency under load is several hundred cycles, so every group of operand reads is
       // issued one phase before the MFMAs that consume it: V rows before the weights are
       // formed, the transposed K columns before dz is formed.
@@ -284,6 +300,8 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
     if (++kt > kt_last) break;
   }
 
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  if (pend_ix >= 0 && qvalid && h == 0) gtab[(unsigned)(pend_ix + qrow)] = Cst[w][n];
   lds_barrier();   // every wave is done with the K/V tiles: their memory becomes the dq staging area
   store_block32<D>(Ks + w * 32 * D, dqacc, a.inv_temp, dqb, a.dq.st, qw0, t.doc_len, lane);
 }
@@ -374,8 +392,8 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     // first steps of the later blocks, fall into the preceding block's rows: in bounds, unused.)
     const int tblock = min((BKV / 32) * kt + sb, (t.doc_len - 1) / 32);
     const int64_t tab_row0 = (int64_t)head * a.tab_stride + t.tab_base;
-    const int64_t tab = tab_row0 + tab_seg(t.doc_len, tblock);
-    const int64_t tab_rowval = tab_row0 + tab_rowplane(t.doc_len);   // per-row plane: rem (stick table), d(rem) (gradient table, written by the dq pass)
+    const int64_t tab = tab_row0 + tab_seg32(t.doc_len, tblock);
+    const int64_t tab_rowval = tab_row0 + tab_rowplane32(t.doc_len);   // per-row plane: rem (stick table), d(rem) (gradient table, written by the dq pass)
     // Fused output o + rem * v: its gradient reaches v_j directly as rem_j * do_j.  The queries of
     // step `sb` are this wave's own keys, so that term is dv = P^T dO with rem_j added on the
     // diagonal of P (which is otherwise zero, or p_jj with attend_current), at no extra traffic.

@@ -55,6 +55,10 @@ __host__ __device__ inline long long tab_block_off(int L, int b) { return (long 
 __host__ __device__ inline long long tab_seg(int L, int b) { return tab_block_off(L, b) - 32ll * b; }
 __host__ __device__ inline long long tab_rowplane(int L) { return tab_block_off(L, (L + 31) / 32); }
 __host__ __device__ inline long long tab_doc_entries(int L) { return tab_rowplane(L) + L; }
+// The same offsets inside ONE document's area as 32-bit values (the scheduler refuses inputs whose
+// tables exceed 2^31 - 1 entries per head): kernels address  uniform base + 32-bit lane offset.
+__device__ __forceinline__ int tab_seg32(int L, int b) { return b * (L - 16 * (b + 1)); }
+__device__ __forceinline__ int tab_rowplane32(int L) { const int nb = (L + 31) >> 5; return nb * L - 16 * nb * (nb - 1); }
 
 struct View {
   char* ptr;
@@ -235,60 +239,54 @@ __device__ __forceinline__ void stick_weights(const f32x16& x, float c, int k0, 
 // Forward-only form of the product-space weights with a quarter of the reciprocals.
 //
 // With e = 2^z (the odds of taking the stick) and t = 1 + e, a key divides the stick by t and
-// takes the difference.  For a group of four keys only ONE reciprocal is needed: the stick
-// after the group's oldest key is (stick before the group) / (t0 t1 t2 t3), and the stick after
-// key i of the group is that times the t of the group's older keys (a running product).  A transcendental costs about four ordinary instructions on this machine, so
-// 16 exp2 + 4 rcp per lane beat 16 exp2 + 16 rcp although a few more multiplies are needed.
+// takes the difference: if A is the stick left on a key's older side, the stick on its newer
+// side is A t and the key's weight is A t - A = A e -- a product, no cancellation.  For a group of
+// four keys only ONE reciprocal is needed: the stick after the group's oldest key is (stick
+// before the group) / (t0 t1 t2 t3); from there the group is walked towards its newest key with
+// p_j = A_j e_j and A_{j+1} = A_j + p_j.  A transcendental costs about four ordinary
+// instructions on this machine, so 16 exp2 + 4 rcp per lane beat 16 exp2 + 16 rcp.
 // The backward kernels need r = 1/t for every key and keep the plain form (stick_weights).
 //
 // The odds are clamped at 2^30 so that a product of four t stays finite (beta = 1 - 2^-30 there,
-// which in fp32 is 1); a masked key has e = 0: t = 1, p = 0.
+// which in fp32 is 1); a masked key has e = 0: its weight is exactly zero and it leaves the
+// stick exactly as it was, so that nothing of a later token reaches the row.
 // ---------------------------------------------------------------------------------------------
 template <bool AC, bool BAND>
 __device__ __forceinline__ void stick_weights_fwd(const f32x16& x, float c, int k0, int qrow, int h,
                                                   float& carry, float (&p)[16]) {
   const int lim = qrow - k0 - 16 * h + (AC ? 1 : 0);   // visible keys of a band block: i < lim
   // per group of four keys (register i = key 16*h + i, so a smaller i is an older key):
-  // u1, u2, u3 = running products of t from the oldest key, inv = 1 / (product of all four)
-  float u1[4], u2[4], u3[4], inv[4];
+  // the odds e and inv = 1 / ((1 + e0) (1 + e1) (1 + e2) (1 + e3))
+  float e[16], inv[4];
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    float t[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int i = 4 * g + j;
-      const float e = fast_exp2(fminf(c * x[i], 30.0f));
-      t[j] = (BAND && !(i < lim)) ? 1.0f : 1.0f + e;
+      const float ej = fast_exp2(fminf(c * x[i], 30.0f));
+      e[i] = (BAND && !(i < lim)) ? 0.0f : ej;
     }
-    u1[g] = t[0];
-    u2[g] = u1[g] * t[1];
-    u3[g] = u2[g] * t[2];
-    inv[g] = fast_rcp(u3[g] * t[3]);
+    float u = 1.0f + e[4 * g];
+    u = fmaf(u, e[4 * g + 1], u);
+    u = fmaf(u, e[4 * g + 2], u);
+    u = fmaf(u, e[4 * g + 3], u);
+    inv[g] = fast_rcp(u);
   }
   const float total = (inv[0] * inv[1]) * (inv[2] * inv[3]);   // what this lane's 16 keys leave of a stick
   float lo, hi;
   both_halves(total, lo, hi);
   // keys of the h=1 lane (16..31) are newer than those of the h=0 lane
   float s = h == 0 ? carry * hi : carry;
-  // Newest group first.  With s the stick after the group's oldest key, the stick after key j
-  // of the group is s * u_j and the stick before its newest key is the previous s; a key's
-  // weight is the difference of the stick before and after it.
+  // Newest group first: s becomes the stick on the older side of the group's oldest key.
 #pragma unroll
   for (int g = 3; g >= 0; --g) {
-    const float before = s;
     s *= inv[g];
-    const float a1 = s * u1[g], a2 = s * u2[g], a3 = s * u3[g];
-    p[4 * g] = a1 - s;
-    p[4 * g + 1] = a2 - a1;
-    p[4 * g + 2] = a3 - a2;
-    p[4 * g + 3] = before - a3;
-  }
-  if (BAND) {
-    // A masked key leaves the stick as it was, but s * (1/u) * u only equals s to rounding:
-    // make its weight exactly zero so that nothing of a later token reaches this row.
+    float a = s;
 #pragma unroll
-    for (int i = 0; i < 16; ++i)
-      if (!(i < lim)) p[i] = 0.0f;
+    for (int j = 0; j < 4; ++j) {
+      p[4 * g + j] = a * e[4 * g + j];
+      if (j < 3) a += p[4 * g + j];
+    }
   }
   carry *= lo * hi;
 }
@@ -425,37 +423,46 @@ __device__ __forceinline__ int swz_off(int row, int chunk) {   // element offset
 // so the swizzle (and the key permutation of key tiles) is applied on the GLOBAL side by
 // choosing which chunk a lane fetches; rows past the end of the document arrive as zeros.
 // Completion is tracked by vmcnt: wait for it, then barrier, before any wave reads the tile.
-// The per-lane part of the source offset is computed once (init); issuing a tile then costs
-// one add per instruction.
+//
+// Instruction j of wave w covers the tile rows  j * STEP + w * RPI .. + RPI - 1  (RPI = rows per
+// instruction, STEP = rows all waves cover together).  STEP is a multiple of 16, which the
+// swizzle does not see, and the key permutation turns "+ STEP rows" into a fixed row offset, so
+// ONE per-lane byte offset serves every instruction: the rest of the address is scalar.
 template <int D, int ROWS, int THREADS, bool KEYS>
 struct TileCopy {
   static constexpr int C8 = D / 8;
   static constexpr int NCH = ROWS * C8 / THREADS;
+  static constexpr int RPI = 64 / C8;                 // rows one wave instruction covers
+  static constexpr int STEP = (THREADS / 64) * RPI;   // rows one instruction of every wave covers
   static_assert(ROWS * C8 % THREADS == 0, "tile must split evenly over the loading threads");
-  int voff[NCH];   // byte offset of this lane's chunk relative to the tile's first row
+  static_assert(STEP % 16 == 0 && (NCH == 1 || STEP == 16 || STEP % 32 == 0), "row step must be invisible to the swizzle");
+  int voff;    // byte offset of this lane's chunk in instruction 0, relative to the tile's first row
   int wave;
+
+  // source row offset of instruction j relative to instruction 0
+  static constexpr int row_delta(int j) {
+    if (!KEYS || STEP % 32 == 0) return j * STEP;
+    // STEP == 16: bit 4 of the tile row becomes bit 3 of the permuted key (see kperm)
+    return 32 * (j >> 1) + 8 * (j & 1);
+  }
 
   // gtid = index of the thread inside the group of THREADS loading threads
   __device__ __forceinline__ void init(int gtid, unsigned row_bytes) {
     wave = __builtin_amdgcn_readfirstlane(gtid >> 6);
     const int lane = gtid & 63;
-#pragma unroll
-    for (int j = 0; j < NCH; ++j) {
-      const int cidx = (wave * NCH + j) * 64 + lane;
-      const int m = cidx / C8, phys = cidx % C8;
-      const int logical = phys ^ swz<D>(m);
-      const int src = KEYS ? ((m & ~31) | kperm(m & 31)) : m;
-      voff[j] = src * (int)row_bytes + logical * 16;
-    }
+    const int m = wave * RPI + lane / C8, phys = lane % C8;
+    const int logical = phys ^ swz<D>(m);
+    const int src = KEYS ? ((m & ~31) | kperm(m & 31)) : m;
+    voff = src * (int)row_bytes + logical * 16;
   }
 
   __device__ __forceinline__ void issue(const Rows& r, int row0, unsigned short* lds_tile) const {
-    const int base = __builtin_amdgcn_readfirstlane(row0 * (int)r.row_bytes);
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
+      const int soff = __builtin_amdgcn_readfirstlane((row0 + row_delta(j)) * (int)r.row_bytes);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          r.rsrc, (__attribute__((address_space(3))) void*)(lds_tile + (wave * NCH + j) * 512), 16,
-          voff[j] + base, 0, 0, 0);
+          r.rsrc, (__attribute__((address_space(3))) void*)(lds_tile + (j * STEP + wave * RPI) * D), 16,
+          voff, soff, 0, 0);
     }
   }
 };

@@ -96,8 +96,8 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
       voff[u][db] = swz_off<D>(r, col >> 3) + (col & 7);
     }
   }
-  // this row's entries of the document's triangular table area
-  float* stick = a.stick == nullptr ? nullptr : a.stick + (int64_t)head * a.tab_stride + t.tab_base + qrow;
+  // the document's triangular table area; a lane adds its row and a block's 32-bit offset
+  float* stick = a.stick == nullptr ? nullptr : a.stick + (int64_t)head * a.tab_stride + t.tab_base;   // (uniform)
 
   // One tile step; the ring slot is a compile-time constant so every LDS address is a fixed
   // register plus an immediate.
@@ -117,7 +117,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
     const int k0 = kt * BF;
     if (sub_skip<AC>(k0, qw0)) return;
     // stick left on entering this block: what both backward kernels start it from
-    if (stick != nullptr && h == 0 && qvalid) stick[tab_seg(t.doc_len, kt)] = carry;
+    if (stick != nullptr && h == 0 && qvalid) stick[(unsigned)(tab_seg32(t.doc_len, kt) + qrow)] = carry;
     f32x16 x;
 #pragma unroll
     for (int i = 0; i < 16; ++i) x[i] = 0.0f;
@@ -179,7 +179,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   if (h == 0 && qvalid) {
     rb[(int64_t)qrow * a.rem.st] = (__bf16)r;
     // rem in full precision for the backward of the fused output (last plane of the table)
-    if (stick != nullptr) stick[tab_rowplane(t.doc_len)] = r;
+    if (stick != nullptr) stick[(unsigned)(tab_rowplane32(t.doc_len) + qrow)] = r;
   }
   lds_barrier();   // every wave is done with the K/V tiles: their memory becomes the o staging area
   if (a.fuse) {
