@@ -324,7 +324,7 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
 // -------------------------------------------------------------------------------------------
 constexpr int NT2 = 512;
 constexpr int BQ = 32;     // queries per step of the dk/dv pass
-constexpr int RING = 8;    // Q/dO tile slots
+constexpr int RING = 6;    // Q/dO tile slots: tiles i-1 (products) .. i+4 (in flight) of step i
 constexpr int AHEAD = 4;   // a tile is requested this many steps before the products use it + 1
 
 template <int D, bool AC, bool PROD>
@@ -449,29 +449,24 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       }
     };
 
-    // Carries are requested three steps ahead and settled two steps ahead, alternating between
-    // two register sets, so a request has two full steps to complete.
-    float carry_e, carry_c, dr, ncarry_e, ncarry_c, ndr;
-    Raw ra, rb;
-    {
-      Raw r0, r1;
-      request(0, r0);
-      request(1, r1);
-      request(2, rb);
-      settle(0, r0, carry_e, carry_c, dr);
-      settle(1, r1, ncarry_e, ncarry_c, ndr);
-    }
+    // Carries are requested three steps before the step that uses them, into three register sets
+    // used in turn (a table read takes longer than one step), and settled when that step begins.
+    float carry_e, carry_c, dr;
+    Raw r0, r1, r2;
+    request(0, r0);
+    request(1, r1);
+    request(2, r2);
     lds_barrier();                        // tiles 0 and 1 are in slots 0 and 1
     // One step: (xc, dc) hold the finished chains of block i; the chains of block i+1 go into
     // (xn, dn).  Called with the two accumulator pairs swapped on alternate steps, so nothing
     // is copied between steps.  DIAG = one of the first steps, whose queries may sit on or
     // above this wave's keys (masks, possible skip); every later step is one straight-line
     // block in which the MFMA chains of block i+1 are interleaved with the VALU work on block i.
-    auto step = [&](auto diag_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& req,
-                    const Raw& due) {
+    auto step = [&](auto diag_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& set) {
       constexpr bool DIAG = decltype(diag_tag)::value;
-      request(i + 3, req);
-      chains((i + 1) & (RING - 1), xn, dn);
+      settle(i, set, carry_e, carry_c, dr);   // requested three steps ago
+      request(i + 3, set);
+      chains((i + 1) % RING, xn, dn);
       bf16x8 pf[2], zf[2];
       const int qw0 = q_first + i * BQ;
       const int qrow = qw0 + n;
@@ -494,9 +489,6 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       }
       stage(i & 1, pf, zf);
       lds_barrier();
-      __builtin_amdgcn_sched_barrier(0);   // keep the consumers of the requested values down here
-      carry_e = ncarry_e; carry_c = ncarry_c; dr = ndr;
-      settle(i + 2, due, ncarry_e, ncarry_c, ndr);   // requested one step ago
     };
     // The same step for the product-space carry away from the diagonal, hand-pipelined: the
     // VALU work on block i is cut into 8 chunks and the 2*KS chain MFMAs of block i+1 are
@@ -505,11 +497,12 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     // SLOT >= 0: the ring slot of tile i+1 (and with it the p/dz buffer, SLOT and i have opposite
     // parity) is a compile-time constant, so every LDS address is a fixed register plus an
     // immediate; SLOT < 0: taken from i at run time.
-    auto bulk = [&](auto slot_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& req, const Raw& due) {
+    auto bulk = [&](auto slot_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& set) {
       constexpr int SLOT = decltype(slot_tag)::value;
       constexpr int NCHUNK = 8, PER = 2 * KS / NCHUNK;
-      request(i + 3, req);
-      const int slot8 = SLOT >= 0 ? SLOT : ((i + 1) & (RING - 1));
+      settle(i, set, carry_e, carry_c, dr);   // requested three steps ago
+      request(i + 3, set);
+      const int slot8 = SLOT >= 0 ? SLOT : ((i + 1) % RING);
       const int parity = SLOT >= 0 ? ((SLOT + 1) & 1) : (i & 1);
       const unsigned short* Qt = Qs + slot8 * QTILE;
       const unsigned short* Gt = Gs + slot8 * QTILE;
@@ -588,46 +581,38 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       stage(parity, pf, zf);
       post(7);
       lds_barrier();
-      __builtin_amdgcn_sched_barrier(0);
-      carry_c = ncarry_c;   // (the running sum of this step ended in registers only)
-      carry_e = ncarry_e; dr = ndr;
-      settle(i + 2, due, ncarry_e, ncarry_c, ndr);
     };
-    auto later = [&](auto slot_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& req, const Raw& due) {
-      if constexpr (PROD) bulk(slot_tag, i, xc, dc, xn, dn, req, due);
-      else step(std::false_type{}, i, xc, dc, xn, dn, req, due);
+    auto later = [&](auto slot_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& set) {
+      if constexpr (PROD) bulk(slot_tag, i, xc, dc, xn, dn, set);
+      else step(std::false_type{}, i, xc, dc, xn, dn, set);
     };
     f32x16 xa, da, xb, db;
     chains(0, xa, da);
-    // the first BKV/BQ steps can touch the diagonal of some wave's block
-    int i = 0;
-#pragma unroll 1
-    for (; i < BKV / BQ && i < nsteps; i += 2) {
-      step(std::true_type{}, i, xa, da, xb, db, ra, rb);
-      if (i + 1 < nsteps) step(std::true_type{}, i + 1, xb, db, xa, da, rb, ra);
-    }
-    // Whole turns of the ring with static slots (i is a multiple of BKV/BQ = 4 here, so tile
-    // i+1 sits in slot 5, 6, 7, 0, ...), then the remaining steps with run-time slots.
+    // the first BKV/BQ = 4 steps can touch the diagonal of some wave's block
+    step(std::true_type{}, 0, xa, da, xb, db, r0);
+    if (nsteps > 1) step(std::true_type{}, 1, xb, db, xa, da, r1);
+    if (nsteps > 2) step(std::true_type{}, 2, xa, da, xb, db, r2);
+    if (nsteps > 3) step(std::true_type{}, 3, xb, db, xa, da, r0);
+    // Whole turns of the ring with static slots (the ring, the two staging buffers, the two
+    // accumulator pairs and the three carry sets all repeat with period six: at i = 4 + 6m tile
+    // i+1 sits in slot 5 and the carries in set 1), then the remaining steps with run-time slots.
     using std::integral_constant;
-    if (i == BKV / BQ) {
+    int i = BKV / BQ;
 #pragma unroll 1
-      for (; i + RING <= nsteps; i += RING) {
-        later(integral_constant<int, 5>{}, i, xa, da, xb, db, ra, rb);
-        later(integral_constant<int, 6>{}, i + 1, xb, db, xa, da, rb, ra);
-        later(integral_constant<int, 7>{}, i + 2, xa, da, xb, db, ra, rb);
-        later(integral_constant<int, 0>{}, i + 3, xb, db, xa, da, rb, ra);
-        later(integral_constant<int, 1>{}, i + 4, xa, da, xb, db, ra, rb);
-        later(integral_constant<int, 2>{}, i + 5, xb, db, xa, da, rb, ra);
-        later(integral_constant<int, 3>{}, i + 6, xa, da, xb, db, ra, rb);
-        later(integral_constant<int, 4>{}, i + 7, xb, db, xa, da, rb, ra);
-      }
+    for (; i + RING <= nsteps; i += RING) {
+      later(integral_constant<int, 5>{}, i, xa, da, xb, db, r1);
+      later(integral_constant<int, 0>{}, i + 1, xb, db, xa, da, r2);
+      later(integral_constant<int, 1>{}, i + 2, xa, da, xb, db, r0);
+      later(integral_constant<int, 2>{}, i + 3, xb, db, xa, da, r1);
+      later(integral_constant<int, 3>{}, i + 4, xa, da, xb, db, r2);
+      later(integral_constant<int, 4>{}, i + 5, xb, db, xa, da, r0);
     }
-#pragma unroll 1
-    for (; i + 1 < nsteps; i += 2) {
-      later(integral_constant<int, -1>{}, i, xa, da, xb, db, ra, rb);
-      later(integral_constant<int, -1>{}, i + 1, xb, db, xa, da, rb, ra);
-    }
-    if (i < nsteps) later(integral_constant<int, -1>{}, i, xa, da, xb, db, ra, rb);
+    // (i = 4 + 6m here: accumulator pair a and carry set 1 are next)
+    if (i < nsteps) later(integral_constant<int, -1>{}, i, xa, da, xb, db, r1);
+    if (i + 1 < nsteps) later(integral_constant<int, -1>{}, i + 1, xb, db, xa, da, r2);
+    if (i + 2 < nsteps) later(integral_constant<int, -1>{}, i + 2, xa, da, xb, db, r0);
+    if (i + 3 < nsteps) later(integral_constant<int, -1>{}, i + 3, xb, db, xa, da, r1);
+    if (i + 4 < nsteps) later(integral_constant<int, -1>{}, i + 4, xa, da, xb, db, r2);
     lds_barrier();                        // the product waves' last step
   } else {
     __builtin_amdgcn_s_setprio(0);
@@ -665,8 +650,8 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     qcopy.init(ptid, qrows.row_bytes);
     gcopy.init(ptid, grows.row_bytes);
     auto fetch = [&](int step) {
-      qcopy.issue(qrows, q_first + step * BQ, Qs + (step & (RING - 1)) * QTILE);
-      gcopy.issue(grows, q_first + step * BQ, Gs + (step & (RING - 1)) * QTILE);
+      qcopy.issue(qrows, q_first + step * BQ, Qs + (step % RING) * QTILE);
+      gcopy.issue(grows, q_first + step * BQ, Gs + (step % RING) * QTILE);
     };
 #pragma unroll
     for (int sft = 0; sft < AHEAD; ++sft)
@@ -678,7 +663,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       if (i >= 1) {
         // acc[key, d] += sum over the 32 queries of step i-1 of X[query][key] * Y[query][d]
         const unsigned short* Xt = (mat ? Zs : Ps) + ((i - 1) & 1) * PTILE;
-        const unsigned short* Yt = (mat ? Qs : Gs) + ((i - 1) & (RING - 1)) * QTILE;
+        const unsigned short* Yt = (mat ? Qs : Gs) + ((i - 1) % RING) * QTILE;
         // operand reads of both contraction steps first, then their products
         bf16x8 af[2][2], bf[2][DB];
 #pragma unroll
