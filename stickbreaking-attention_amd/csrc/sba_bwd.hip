@@ -529,24 +529,25 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
         }
         __builtin_amdgcn_sched_barrier(0);
       };
-      pre(0);
-      pre(1);
+      // The step opens with vector work only: right after the barrier the product waves fetch the
+      // p / dz fragments this wave's neighbours just staged, and they are the ones the next barrier
+      // waits for -- the score waves' own operand reads join one chunk later.
       float r[16], ex[16], p[16];
       // chunks 0, 1: r = 1 - beta of the 16 keys
-      pre(2);
 #pragma unroll
       for (int j = 0; j < 8; ++j) r[j] = fast_rcp(1.0f + fast_exp2(a.c * xc[j]));
-      post(0);
-      pre(3);
+      __builtin_amdgcn_sched_barrier(0);
+      pre(0);
+      pre(1);
 #pragma unroll
       for (int j = 8; j < 16; ++j) r[j] = fast_rcp(1.0f + fast_exp2(a.c * xc[j]));
-      post(1);
+      __builtin_amdgcn_sched_barrier(0);
       // chunk 2: stick left after the newer keys
-      pre(4);
+      pre(2);
       carry_e = suffix_prod32_excl(r, ex, h, carry_e);
-      post(2);
+      post(0);
       // chunk 3: weights and their bf16 fragments
-      pre(5);
+      pre(3);
       const float after = ex[0] * r[0];       // stick left after this lane's oldest key
       p[0] = ex[0] - after;
 #pragma unroll
@@ -554,9 +555,9 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       bf16x8 pf[2], zf[2];
       pf[0] = pack8(p);
       pf[1] = pack8(p + 8);
-      post(3);
+      post(1);
       // chunk 4: this lane's total of G = sum(p do.v) - drem sum(p), sum(p) = ex[15] - after
-      pre(4 + LEAD);
+      pre(4);
       float t0 = 0.0f, t1 = 0.0f;
 #pragma unroll
       for (int j = 0; j < 16; j += 2) { t0 = fmaf(p[j], dc[j], t0); t1 = fmaf(p[j + 1], dc[j + 1], t1); }
@@ -564,21 +565,23 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       both_halves(fmaf(-dr, ex[15] - after, t0 + t1), lo, hi);
       // chunks 5, 6: D = C + drem * stick runs on do.v directly (see grad_dz); dz = r D[i] - D[i-1]
       float dprev = fmaf(dr, after, h == 1 ? carry_c + lo : carry_c);
-      post(4);
+      post(2);
       float dz[16];
-      pre(5 + LEAD);
+      pre(5);
 #pragma unroll
       for (int j = 0; j < 8; ++j) { const float dj = fmaf(p[j], dc[j], dprev); dz[j] = fmaf(r[j], dj, -dprev); dprev = dj; }
-      post(5);
-      pre(6 + LEAD);
+      post(3);
+      pre(6);
 #pragma unroll
       for (int j = 8; j < 16; ++j) { const float dj = fmaf(p[j], dc[j], dprev); dz[j] = fmaf(r[j], dj, -dprev); dprev = dj; }
-      post(6);
+      post(4);
       // chunk 7: dz fragments and staging
-      pre(9);
+      pre(7);
       zf[0] = pack8(dz);
       zf[1] = pack8(dz + 8);
       stage(parity, pf, zf);
+      post(5);
+      post(6);
       post(7);
       lds_barrier();
     };
@@ -658,31 +661,17 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       if (sft < nsteps) fetch(sft);
     wait_loads<0>();
     lds_barrier();
-    for (int i = 0; i <= nsteps; ++i) {
-      if (i + AHEAD < nsteps) fetch(i + AHEAD);
-      if (i >= 1) {
-        // acc[key, d] += sum over the 32 queries of step i-1 of X[query][key] * Y[query][d]
-        const unsigned short* Xt = (mat ? Zs : Ps) + ((i - 1) & 1) * PTILE;
-        const unsigned short* Yt = (mat ? Qs : Gs) + ((i - 1) % RING) * QTILE;
-        // operand reads of both contraction steps first, then their products
-        bf16x8 af[2][2], bf[2][DB];
+    // The LDS is the busiest unit of this kernel (every step moves about 140 KB through it), and
+    // a product wave that fetched all its operands after the barrier would spend half the step
+    // issuing reads.  Only the staged p / dz fragments have to wait for the barrier: the Q / dO
+    // fragments of a step come from a tile that landed long before, so they are read one
+    // iteration ahead, between the MFMAs of the previous step.
+    auto read_y = [&](int step, bf16x8 (&bf)[2][DB], int ks) {
+      const unsigned short* Yt = (mat ? Qs : Gs) + (step % RING) * QTILE;
 #pragma unroll
-        for (int ks = 0; ks < BQ / 16; ++ks) {
-#pragma unroll
-          for (int kb2 = 0; kb2 < 2; ++kb2)
-            af[ks][kb2] = lds_tr8(Xt + xoff[0][kb2] + 16 * ks * BKV, Xt + xoff[1][kb2] + 16 * ks * BKV);
-#pragma unroll
-          for (int j = 0; j < DB; ++j)
-            bf[ks][j] = lds_tr8(Yt + yoff[0][j] + 16 * ks * D, Yt + yoff[1][j] + 16 * ks * D);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ks = 0; ks < BQ / 16; ++ks)
-#pragma unroll
-          for (int kb2 = 0; kb2 < 2; ++kb2)
-#pragma unroll
-            for (int j = 0; j < DB; ++j) acc[kb2][j] = mfma32(af[ks][kb2], bf[ks][j], acc[kb2][j]);
-      }
+      for (int j = 0; j < DB; ++j) bf[ks][j] = lds_tr8(Yt + yoff[0][j] + 16 * ks * D, Yt + yoff[1][j] + 16 * ks * D);
+    };
+    auto finish = [&](int i) {
       // Tile i+2 (read by the score waves in step i+1) has landed before anyone passes the
       // barrier: only the tiles requested after it may still be in flight (loads return in order).
       const int after = min(i + AHEAD, nsteps - 1) - (i + 2);
@@ -690,6 +679,39 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       else if (after == 1) wait_loads<LOADS_PER_TILE>();
       else wait_loads<0>();
       lds_barrier();
+    };
+    // iteration i >= 1: products of step i - 1 with the Q / dO fragments in `cur`; the fragments of
+    // step i go into `nxt` (past the last step they come from an idle ring slot and are never used)
+    auto iter = [&](int i, bf16x8 (&cur)[2][DB], bf16x8 (&nxt)[2][DB]) {
+      if (i + AHEAD < nsteps) fetch(i + AHEAD);
+      // acc[key, d] += sum over the 32 queries of step i-1 of X[query][key] * Y[query][d]
+      const unsigned short* Xt = (mat ? Zs : Ps) + ((i - 1) & 1) * PTILE;
+      bf16x8 af[2][2];
+#pragma unroll
+      for (int ks = 0; ks < BQ / 16; ++ks)
+#pragma unroll
+        for (int kb2 = 0; kb2 < 2; ++kb2)
+          af[ks][kb2] = lds_tr8(Xt + xoff[0][kb2] + 16 * ks * BKV, Xt + xoff[1][kb2] + 16 * ks * BKV);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 0; ks < BQ / 16; ++ks) {
+#pragma unroll
+        for (int kb2 = 0; kb2 < 2; ++kb2)
+#pragma unroll
+          for (int j = 0; j < DB; ++j) acc[kb2][j] = mfma32(af[ks][kb2], cur[ks][j], acc[kb2][j]);
+        read_y(i, nxt, ks);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      finish(i);
+    };
+    bf16x8 ya[2][DB], yb[2][DB];
+    if (AHEAD < nsteps) fetch(AHEAD);
+    read_y(0, ya, 0);
+    read_y(0, ya, 1);
+    finish(0);
+    for (int i = 1; i <= nsteps; i += 2) {
+      iter(i, ya, yb);
+      if (i + 1 <= nsteps) iter(i + 1, yb, ya);
     }
     // (the last barrier of the loop has passed: the p/dz staging buffers are free)
     const View& ov = mat ? a.dk : a.dv;
