@@ -44,13 +44,17 @@ int check_problem(const sba_problem* p, bool fixed, Sizes* sz) {
 }
 
 // Carry-table entries per head.  Fixed-length: exact.  Packed documents: the most any split of
-// `tokens` tokens into documents of at most max_doc_len tokens can need (the per-document need is
-// convex in the length, so the worst split is as many longest documents as fit plus the rest).
+// `tokens` tokens into n_docs documents of at most max_doc_len tokens can need.  A document
+// occupies what its length rounded up to a multiple of 32 needs, and that need is convex in
+// the length, so the worst split is as many longest documents as fit plus the rest, with every
+// document's rounding (at most 31 tokens each) added to the token count.
 long long table_entries_bound(const sba_problem* p, bool fixed) {
   if (fixed) return (long long)p->batch * tab_doc_entries(p->tokens);
-  const int lmax = (p->max_doc_len > 0 && p->max_doc_len < p->tokens) ? p->max_doc_len : p->tokens;
+  const long long tokens = (long long)p->tokens + 31ll * p->n_docs;
+  long long lmax = (p->max_doc_len > 0 && p->max_doc_len < p->tokens) ? p->max_doc_len : p->tokens;
+  lmax = (lmax + 31) & ~31ll;
   if (lmax <= 0) return 0;
-  return (long long)(p->tokens / lmax) * tab_doc_entries(lmax) + tab_doc_entries(p->tokens % lmax);
+  return (tokens / lmax) * tab_doc_entries((int)lmax) + tab_doc_entries((int)(tokens % lmax));
 }
 
 size_t schedule_bytes(const Sizes& sz) {
@@ -126,7 +130,7 @@ int fill_common(const sba_problem* p, bool fixed, const Sizes& sz, const void* s
   if (sched_bytes < schedule_bytes(sz)) return SBA_E_WORKSPACE;
   a->tab_stride = -1;
   if (with_table) {
-    a->tab_stride = (int64_t)(table_bytes / sizeof(float) / (size_t)p->heads);
+    a->tab_stride = (int64_t)(table_bytes / sizeof(float) / (size_t)p->heads) & ~(int64_t)31;   // heads start on 128-byte lines
     // fixed-length needs are known here; packed documents are checked on the device against
     // what the scheduler found (kernels refuse to run, outputs are filled with NaN)
     if (fixed && a->tab_stride < table_entries_bound(p, true)) return SBA_E_WORKSPACE;
@@ -291,7 +295,7 @@ size_t sba_table_bytes_for_lengths(const sba_problem* p, const int64_t* doc_leng
     entries += tab_doc_entries((int)doc_lengths[i]);
   }
   if (entries > 0x7fffffffll) return 0;   // a document's base must fit the scheduler's int32 field
-  return (size_t)p->heads * (size_t)(entries > 0 ? entries : 1) * sizeof(float);
+  return (size_t)p->heads * (size_t)(entries > 0 ? entries : 32) * sizeof(float);   // never empty: one 128-byte line per head
 }
 
 int sba_build_schedule(const sba_problem* p, void* schedule, size_t schedule_size, void* stream) {

@@ -47,18 +47,19 @@ struct Tile {
 };
 
 // Carry tables (fp32).  Inside a head's share every document owns a triangular area: for each
-// 32-key block b the rows 32*b .. L-1 (the queries at or below the block), blocks back to back,
-// then one plane of L per-row values.  Entry (b, row) sits at  tab_seg(L, b) + row  from the
-// document's base: consecutive rows are consecutive floats, so the 32 lanes that own 32
-// consecutive query rows read and write 128 contiguous bytes.
-__host__ __device__ inline long long tab_block_off(int L, int b) { return (long long)b * L - 16ll * b * (b - 1); }
+// 32-key block b the rows 32*b .. Lp-1 (the queries at or below the block; Lp = the length
+// rounded up to a multiple of 32), blocks back to back, then one plane of Lp per-row values.
+// Entry (b, row) sits at  tab_seg(L, b) + row  from the document's base: consecutive rows are
+// consecutive floats and every block's rows start on a 128-byte boundary, so the 32 lanes that
+// own 32 consecutive query rows read and write one aligned 128-byte line.
+__host__ __device__ inline long long tab_block_off(int L, int b) { return 32ll * b * ((L + 31) >> 5) - 16ll * b * (b - 1); }
 __host__ __device__ inline long long tab_seg(int L, int b) { return tab_block_off(L, b) - 32ll * b; }
-__host__ __device__ inline long long tab_rowplane(int L) { return tab_block_off(L, (L + 31) / 32); }
-__host__ __device__ inline long long tab_doc_entries(int L) { return tab_rowplane(L) + L; }
+__host__ __device__ inline long long tab_rowplane(int L) { return tab_block_off(L, (L + 31) >> 5); }
+__host__ __device__ inline long long tab_doc_entries(int L) { return tab_rowplane(L) + 32ll * ((L + 31) >> 5); }
 // The same offsets inside ONE document's area as 32-bit values (the scheduler refuses inputs whose
 // tables exceed 2^31 - 1 entries per head): kernels address  uniform base + 32-bit lane offset.
-__device__ __forceinline__ int tab_seg32(int L, int b) { return b * (L - 16 * (b + 1)); }
-__device__ __forceinline__ int tab_rowplane32(int L) { const int nb = (L + 31) >> 5; return nb * L - 16 * nb * (nb - 1); }
+__device__ __forceinline__ int tab_seg32(int L, int b) { return b * (32 * ((L + 31) >> 5) - 16 * (b + 1)); }
+__device__ __forceinline__ int tab_rowplane32(int L) { const int nb = (L + 31) >> 5; return 16 * nb * (nb + 1); }
 
 struct View {
   char* ptr;

@@ -54,18 +54,21 @@ def _padded_dim(d: int) -> int:
 
 
 def table_entries(length: int) -> int:
-    """Carry-table entries one document of `length` tokens needs per head: one per (32-key block,
-    query row at or below it) pair plus one per row (``tab_doc_entries`` in csrc/sba_device.hpp)."""
+    """Carry-table entries one document of `length` tokens needs per head: with the length rounded up
+    to a multiple of 32, one per (32-key block, query row at or below it) pair plus one per row
+    (``tab_doc_entries`` in csrc/sba_device.hpp)."""
     nb = -(-length // _BT)
-    return nb * length - 16 * nb * (nb - 1) + length
+    return 16 * nb * (nb + 1) + 32 * nb
 
 
-def table_entries_bound(tokens: int, max_doc_len: int) -> int:
-    """The most any split of `tokens` tokens into documents of at most `max_doc_len` can need."""
+def table_entries_bound(tokens: int, max_doc_len: int, n_docs: int) -> int:
+    """The most any split of `tokens` tokens into `n_docs` documents of at most `max_doc_len` can need."""
     lmax = max_doc_len if 0 < max_doc_len < tokens else tokens
+    lmax = (lmax + 31) & ~31
     if lmax <= 0:
         return 0
-    return (tokens // lmax) * table_entries(lmax) + table_entries(tokens % lmax)
+    padded = tokens + 31 * n_docs
+    return (padded // lmax) * table_entries(lmax) + table_entries(padded % lmax)
 
 
 def workspace_sizes(fixed: bool, batch: int, heads: int, tokens: int, n_docs: int, max_doc_len: int,
@@ -82,9 +85,9 @@ def workspace_sizes(fixed: bool, batch: int, heads: int, tokens: int, n_docs: in
     if fixed:
         entries = batch * table_entries(tokens)
     elif lengths is not None:
-        entries = max(1, sum(table_entries(int(n)) for n in lengths))
+        entries = max(32, sum(table_entries(int(n)) for n in lengths))
     else:
-        entries = table_entries_bound(tokens, max_doc_len)
+        entries = table_entries_bound(tokens, max_doc_len, n_docs)
     return (4 * words + 255) & ~255, heads * entries
 
 
