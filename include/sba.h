@@ -107,7 +107,8 @@ typedef struct sba_problem {
 size_t sba_schedule_bytes(const sba_problem* p);
 
 /* Bytes of ONE carry table.  A table holds, per head and per document of length L, one fp32 for
- * every (32-key block, query row at or below it) pair -- about L*L/64 -- plus one per row (the
+ * every (32-key block, query row at or below it) pair -- about L*L/64, L rounded up to a
+ * multiple of 32 so that every block starts on a 128-byte line -- plus one per row (the
  * forward leaves rem there in fp32, the backward the complete gradient of rem).  The forward
  * fills `stick_table`; the backward additionally needs a `grad_table` of the same size.
  *   sba_table_bytes              no lengths needed: the most any documents of at most
