@@ -39,12 +39,12 @@
 extern "C" {
 #endif
 
-#define SBA_VERSION 201
+#define SBA_VERSION 202
 
 /* error codes (negative returns) */
 #define SBA_E_NULL      (-1)  /* a required pointer is NULL                         */
 #define SBA_E_HEAD_DIM  (-2)  /* head_dim not in {64, 128}                          */
-#define SBA_E_DTYPE     (-3)  /* dtype not SBA_BF16                                 */
+#define SBA_E_DTYPE     (-3)  /* dtype neither SBA_BF16 nor SBA_F16                 */
 #define SBA_E_SHAPE     (-4)  /* negative / inconsistent sizes, or tokens*stride_t
                                  too large for 32-bit byte offsets (>= 2 GiB)       */
 #define SBA_E_STRIDE    (-5)  /* a row start is not 16-byte aligned (stride % 8)    */
@@ -54,8 +54,10 @@ extern "C" {
                                  sba_varlen_fwd_static                              */
 #define SBA_E_ARCH      (-7)  /* current device is not gfx950                       */
 
-/* element types */
+/* element types of q, k, v, grad_o, grad_rem and of every output (one type per call); the
+ * matrix products run on the MFMA instruction of that type with fp32 accumulation */
 #define SBA_BF16 1
+#define SBA_F16  2
 
 /* flags */
 #define SBA_ATTEND_CURRENT 1u   /* a token may attend to itself (upstream attend_current) */
@@ -85,7 +87,7 @@ typedef struct sba_view {
 
 /* Problem description shared by all entry points. */
 typedef struct sba_problem {
-  int32_t  dtype;        /* SBA_BF16                                                     */
+  int32_t  dtype;        /* SBA_BF16 or SBA_F16                                          */
   int32_t  head_dim;     /* 64 or 128                                                    */
   int32_t  heads;        /* H                                                            */
   int32_t  batch;        /* B for the fixed-length op, 1 for varlen                      */

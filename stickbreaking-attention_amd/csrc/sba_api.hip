@@ -26,7 +26,7 @@ struct Sizes {
 
 int check_problem(const sba_problem* p, bool fixed, Sizes* sz) {
   if (p == nullptr) return SBA_E_NULL;
-  if (p->dtype != SBA_BF16) return SBA_E_DTYPE;
+  if (p->dtype != SBA_BF16 && p->dtype != SBA_F16) return SBA_E_DTYPE;
   if (p->head_dim != 64 && p->head_dim != 128) return SBA_E_HEAD_DIM;
   if (p->heads <= 0 || p->tokens < 0 || p->batch <= 0 || p->max_doc_len < 0) return SBA_E_SHAPE;
   if (fixed != ((p->flags & SBA_FIXED_LENGTH) != 0)) return SBA_E_SHAPE;
@@ -169,7 +169,7 @@ int forward(const sba_problem* p, bool fixed, const void* schedule, size_t sched
   hipError_t he = hipSuccess;
   if (sz.n_docs > 0) {
     Timer tm(0, s, timed);
-    he = launch_fwd(a, p->head_dim, (p->flags & SBA_ATTEND_CURRENT) != 0,
+    he = (p->dtype == SBA_F16 ? f16::launch_fwd : bf16::launch_fwd)(a, p->head_dim, (p->flags & SBA_ATTEND_CURRENT) != 0,
                     (p->flags & SBA_PRODUCT_SPACE) != 0, weights != nullptr, sz.n_q_max, s);
   }
   if (he != hipSuccess || fixed) return (int)he;
@@ -178,6 +178,7 @@ int forward(const sba_problem* p, bool fixed, const void* schedule, size_t sched
   z.mat[0] = a.o; z.n_mat = 1; z.row = a.rem;
   z.sched = a.sched; z.heads = p->heads; z.tokens = p->tokens; z.head_dim = p->head_dim;
   z.tab_stride = a.tab_stride;
+  z.nan_pair = p->dtype == SBA_F16 ? 0x7e007e00u : 0x7fc07fc0u;
   return (int)launch_zero_tail(z, s);
 }
 
@@ -208,12 +209,12 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, size_t sche
   if (sz.n_docs > 0) {
     {
       Timer tm(1, s);
-      he = launch_bwd_dq(a, p->head_dim, ac, prod, sz.n_q_max, s);
+      he = (p->dtype == SBA_F16 ? f16::launch_bwd_dq : bf16::launch_bwd_dq)(a, p->head_dim, ac, prod, sz.n_q_max, s);
     }
     if (he != hipSuccess) return (int)he;
     {
       Timer tm(2, s);
-      he = launch_bwd_dkdv(a, p->head_dim, ac, prod, sz.n_kv_max, s);
+      he = (p->dtype == SBA_F16 ? f16::launch_bwd_dkdv : bf16::launch_bwd_dkdv)(a, p->head_dim, ac, prod, sz.n_kv_max, s);
     }
   }
   if (he != hipSuccess || fixed) return (int)he;
@@ -222,6 +223,7 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, size_t sche
   z.mat[0] = a.dq; z.mat[1] = a.dk; z.mat[2] = a.dv; z.n_mat = 3;
   z.sched = a.sched; z.heads = p->heads; z.tokens = p->tokens; z.head_dim = p->head_dim;
   z.tab_stride = a.tab_stride;
+  z.nan_pair = p->dtype == SBA_F16 ? 0x7e007e00u : 0x7fc07fc0u;
   return (int)launch_zero_tail(z, s);
 }
 
@@ -261,7 +263,7 @@ const char* sba_error_string(int code) {
     case 0: return "ok";
     case SBA_E_NULL: return "a required pointer is NULL";
     case SBA_E_HEAD_DIM: return "head_dim must be 64 or 128";
-    case SBA_E_DTYPE: return "unsupported element type (bf16 only)";
+    case SBA_E_DTYPE: return "unsupported element type (SBA_BF16 or SBA_F16)";
     case SBA_E_SHAPE: return "negative or inconsistent sizes";
     case SBA_E_STRIDE: return "pointer or stride breaks 16-byte row alignment";
     case SBA_E_WORKSPACE: return "workspace too small";

@@ -24,6 +24,7 @@
 #include "sba_kernels.hpp"
 
 namespace sba {
+inline namespace SBA_ELEM_NS {
 
 // One 32-key sub-block for the 32 queries of a wave, in two phases so that the do.v^T
 // accumulators need not be live while the weights are formed:
@@ -56,7 +57,7 @@ __device__ __forceinline__ void grad_weights(const f32x16& x, float c, int k0, i
 template <bool PROD>
 __device__ __forceinline__ void grad_dz(const float (&p)[16], const float (&r)[16], const f32x16& da,
                                         const float (&ends)[2], int h, float& carry_c, float dr,
-                                        bf16x8 (&zf)[2]) {
+                                        el8 (&zf)[2]) {
   float dz[16];
   if constexpr (PROD) {
     float t0 = 0.0f, t1 = 0.0f;
@@ -129,11 +130,11 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   const bool qvalid = qrow < t.doc_len;
 
   const int64_t tok0 = t.tok_start;
-  const __bf16* qb = reinterpret_cast<const __bf16*>(a.q.ptr) + t.batch * a.q.sb + head * a.q.sh + tok0 * a.q.st;
-  const __bf16* kb = reinterpret_cast<const __bf16*>(a.k.ptr) + t.batch * a.k.sb + head * a.k.sh + tok0 * a.k.st;
-  const __bf16* vb = reinterpret_cast<const __bf16*>(a.v.ptr) + t.batch * a.v.sb + head * a.v.sh + tok0 * a.v.st;
-  const __bf16* gob = reinterpret_cast<const __bf16*>(a.go.ptr) + t.batch * a.go.sb + head * a.go.sh + tok0 * a.go.st;
-  __bf16* dqb = reinterpret_cast<__bf16*>(a.dq.ptr) + t.batch * a.dq.sb + head * a.dq.sh + tok0 * a.dq.st;
+  const elem_t* qb = reinterpret_cast<const elem_t*>(a.q.ptr) + t.batch * a.q.sb + head * a.q.sh + tok0 * a.q.st;
+  const elem_t* kb = reinterpret_cast<const elem_t*>(a.k.ptr) + t.batch * a.k.sb + head * a.k.sh + tok0 * a.k.st;
+  const elem_t* vb = reinterpret_cast<const elem_t*>(a.v.ptr) + t.batch * a.v.sb + head * a.v.sh + tok0 * a.v.st;
+  const elem_t* gob = reinterpret_cast<const elem_t*>(a.go.ptr) + t.batch * a.go.sb + head * a.go.sh + tok0 * a.go.st;
+  elem_t* dqb = reinterpret_cast<elem_t*>(a.dq.ptr) + t.batch * a.dq.sb + head * a.dq.sh + tok0 * a.dq.st;
   const Rows qrows = make_rows(qb, a.q.st, t.doc_len);
   const Rows grows = make_rows(gob, a.go.st, t.doc_len);
   const Rows krows = make_rows(kb, a.k.st, t.doc_len);
@@ -145,7 +146,7 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   kcopy.issue(krows, 0, Ks);
   vcopy.issue(vrows, 0, Vs);
 
-  bf16x8 qf[KS], dof[KS];
+  el8 qf[KS], dof[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     qf[ks] = load_frag(qrows, qrow, 32 * ks + 16 * h);
@@ -155,14 +156,14 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   // that sum also reaches rem, through the row's own value vector: d(rem) += do . v_row.
   float dr = 0.0f;
   if (a.grem.ptr != nullptr && qvalid) {
-    const __bf16* grb = reinterpret_cast<const __bf16*>(a.grem.ptr) + t.batch * a.grem.sb + head * a.grem.sh + tok0 * a.grem.st;
+    const elem_t* grb = reinterpret_cast<const elem_t*>(a.grem.ptr) + t.batch * a.grem.sb + head * a.grem.sh + tok0 * a.grem.st;
     dr = (float)grb[(int64_t)qrow * a.grem.st];
   }
   if (a.fuse) {
     float dot = 0.0f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const bf16x8 vown = load_frag(vrows, qrow, 32 * ks + 16 * h);
+      const el8 vown = load_frag(vrows, qrow, 32 * ks + 16 * h);
 #pragma unroll
       for (int e = 0; e < 8; ++e) dot = fmaf((float)dof[ks][e], (float)vown[e], dot);
     }
@@ -252,12 +253,12 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
       // issued one phase before the MFMAs that consume it: V rows before the weights are
       // formed, the transposed K columns before dz is formed.
       float p[16], bt[16], ends[2] = {0.0f, 0.0f};
-      bf16x8 vfr[KS];
+      el8 vfr[KS];
       {
         f32x16 x;
 #pragma unroll
         for (int i = 0; i < 16; ++i) x[i] = 0.0f;
-        bf16x8 kfr[KS];
+        el8 kfr[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) kfr[ks] = lds_row8(Kt + 32 * sb * D + roff[ks]);
 #pragma unroll
@@ -267,8 +268,8 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         grad_weights<AC, PROD>(x, a.c, k0, qw0, qrow, h, ce[sb], p, bt, ends);
       }
-      bf16x8 zf[2];
-      bf16x8 ktr[2][DB];
+      el8 zf[2];
+      el8 ktr[2][DB];
       {
         f32x16 da;
 #pragma unroll
@@ -358,10 +359,10 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   const bool scorer = w < 4;
 
   const int64_t tok0 = t.tok_start;
-  const __bf16* qb = reinterpret_cast<const __bf16*>(a.q.ptr) + t.batch * a.q.sb + head * a.q.sh + tok0 * a.q.st;
-  const __bf16* kb = reinterpret_cast<const __bf16*>(a.k.ptr) + t.batch * a.k.sb + head * a.k.sh + tok0 * a.k.st;
-  const __bf16* vb = reinterpret_cast<const __bf16*>(a.v.ptr) + t.batch * a.v.sb + head * a.v.sh + tok0 * a.v.st;
-  const __bf16* gob = reinterpret_cast<const __bf16*>(a.go.ptr) + t.batch * a.go.sb + head * a.go.sh + tok0 * a.go.st;
+  const elem_t* qb = reinterpret_cast<const elem_t*>(a.q.ptr) + t.batch * a.q.sb + head * a.q.sh + tok0 * a.q.st;
+  const elem_t* kb = reinterpret_cast<const elem_t*>(a.k.ptr) + t.batch * a.k.sb + head * a.k.sh + tok0 * a.k.st;
+  const elem_t* vb = reinterpret_cast<const elem_t*>(a.v.ptr) + t.batch * a.v.sb + head * a.v.sh + tok0 * a.v.st;
+  const elem_t* gob = reinterpret_cast<const elem_t*>(a.go.ptr) + t.batch * a.go.sb + head * a.go.sh + tok0 * a.go.st;
   const Rows qrows = make_rows(qb, a.q.st, t.doc_len);
   const Rows grows = make_rows(gob, a.go.st, t.doc_len);
   const Rows krows = make_rows(kb, a.k.st, t.doc_len);
@@ -380,7 +381,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     const int sb = w;                           // 32-key block of this wave
     const int k0 = kt * BKV + 32 * sb;
     const int qr = n;                           // this lane's query row inside a tile
-    bf16x8 kf[KS], vf[KS];                      // MFMA row n holds key k0 + kperm(n)
+    el8 kf[KS], vf[KS];                      // MFMA row n holds key k0 + kperm(n)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       kf[ks] = load_frag(krows, k0 + kperm(n), 32 * ks + 16 * h);
@@ -428,7 +429,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
 #pragma unroll
       for (int j = 0; j < 16; ++j) { x[j] = 0.0f; da[j] = 0.0f; }
       // all operand reads first, so the chains are not paced by LDS latency
-      bf16x8 qfr[KS], gfr[KS];
+      el8 qfr[KS], gfr[KS];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) { qfr[ks] = lds_row8(Qt + roff[ks]); gfr[ks] = lds_row8(Gt + roff[ks]); }
 #pragma unroll
@@ -437,15 +438,15 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
         da = mfma32(vf[ks], gfr[ks], da);
       }
     };
-    auto stage = [&](int parity, const bf16x8 (&pf)[2], const bf16x8 (&zf)[2]) {
+    auto stage = [&](int parity, const el8 (&pf)[2], const el8 (&zf)[2]) {
       // p and dz as [query][key]: fragment tt is 8 consecutive keys = one 16-byte chunk
       unsigned short* Pt = Ps + parity * PTILE;
       unsigned short* Zt = Zs + parity * PTILE;
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt) {
         const int chunk = 4 * sb + 2 * h + tt;
-        *reinterpret_cast<bf16x8*>(Pt + swz_off<BKV>(qr, chunk)) = pf[tt];
-        *reinterpret_cast<bf16x8*>(Zt + swz_off<BKV>(qr, chunk)) = zf[tt];
+        *reinterpret_cast<el8*>(Pt + swz_off<BKV>(qr, chunk)) = pf[tt];
+        *reinterpret_cast<el8*>(Zt + swz_off<BKV>(qr, chunk)) = zf[tt];
       }
     };
 
@@ -467,7 +468,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       settle(i, set, carry_e, carry_c, dr);   // requested three steps ago
       request(i + 3, set);
       chains((i + 1) % RING, xn, dn);
-      bf16x8 pf[2], zf[2];
+      el8 pf[2], zf[2];
       const int qw0 = q_first + i * BQ;
       const int qrow = qw0 + n;
       if (DIAG && sub_skip<AC>(k0, qw0)) {
@@ -511,7 +512,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       // Operand reads run LEAD chunks ahead of the MFMAs that consume them (LDS latency under
       // load is longer than one chunk of VALU work), through a small rotating set of registers.
       constexpr int LEAD = 2;
-      bf16x8 fr[LEAD + 1][PER];
+      el8 fr[LEAD + 1][PER];
       auto pre = [&](int c) {
         if (c >= NCHUNK) return;
 #pragma unroll
@@ -552,7 +553,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       p[0] = ex[0] - after;
 #pragma unroll
       for (int j = 1; j < 16; ++j) p[j] = ex[j] - ex[j - 1];
-      bf16x8 pf[2], zf[2];
+      el8 pf[2], zf[2];
       pf[0] = pack8(p);
       pf[1] = pack8(p + 8);
       post(1);
@@ -666,7 +667,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     // issuing reads.  Only the staged p / dz fragments have to wait for the barrier: the Q / dO
     // fragments of a step come from a tile that landed long before, so they are read one
     // iteration ahead, between the MFMAs of the previous step.
-    auto read_y = [&](int step, bf16x8 (&bf)[2][DB], int ks) {
+    auto read_y = [&](int step, el8 (&bf)[2][DB], int ks) {
       const unsigned short* Yt = (mat ? Qs : Gs) + (step % RING) * QTILE;
 #pragma unroll
       for (int j = 0; j < DB; ++j) bf[ks][j] = lds_tr8(Yt + yoff[0][j] + 16 * ks * D, Yt + yoff[1][j] + 16 * ks * D);
@@ -682,11 +683,11 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     };
     // iteration i >= 1: products of step i - 1 with the Q / dO fragments in `cur`; the fragments of
     // step i go into `nxt` (past the last step they come from an idle ring slot and are never used)
-    auto iter = [&](int i, bf16x8 (&cur)[2][DB], bf16x8 (&nxt)[2][DB]) {
+    auto iter = [&](int i, el8 (&cur)[2][DB], el8 (&nxt)[2][DB]) {
       if (i + AHEAD < nsteps) fetch(i + AHEAD);
       // acc[key, d] += sum over the 32 queries of step i-1 of X[query][key] * Y[query][d]
       const unsigned short* Xt = (mat ? Zs : Ps) + ((i - 1) & 1) * PTILE;
-      bf16x8 af[2][2];
+      el8 af[2][2];
 #pragma unroll
       for (int ks = 0; ks < BQ / 16; ++ks)
 #pragma unroll
@@ -704,7 +705,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       }
       finish(i);
     };
-    bf16x8 ya[2][DB], yb[2][DB];
+    el8 ya[2][DB], yb[2][DB];
     if (AHEAD < nsteps) fetch(AHEAD);
     read_y(0, ya, 0);
     read_y(0, ya, 1);
@@ -715,7 +716,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     }
     // (the last barrier of the loop has passed: the p/dz staging buffers are free)
     const View& ov = mat ? a.dk : a.dv;
-    __bf16* outb = reinterpret_cast<__bf16*>(ov.ptr) + t.batch * ov.sb + head * ov.sh + tok0 * ov.st;
+    elem_t* outb = reinterpret_cast<elem_t*>(ov.ptr) + t.batch * ov.sb + head * ov.sh + tok0 * ov.st;
     unsigned short* scratch = (w & 2 ? Zs : Ps) + (w & 1) * 32 * D;
 #pragma unroll
     for (int kb2 = 0; kb2 < 2; ++kb2)
@@ -778,4 +779,5 @@ hipError_t launch_bwd_dkdv(const KArgs& a, int head_dim, bool ac, bool prod, int
   return launch_dkdv_d<64>(a, ac, prod, n_kv_max, s);
 }
 
+}  // inline namespace SBA_ELEM_NS
 }  // namespace sba

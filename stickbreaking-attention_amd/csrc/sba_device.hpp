@@ -11,11 +11,18 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+// The kernels are written once for a 16-bit element type and compiled twice: for bfloat16 (the
+// default) and, with SBA_ELEM_F16 defined, for IEEE half.  Everything that depends on the element
+// type lives in an inline namespace named after it, so the two compilations produce distinct
+// symbols and one library holds both.
+#ifdef SBA_ELEM_F16
+#define SBA_ELEM_NS f16
+#else
+#define SBA_ELEM_NS bf16
+#endif
+
 namespace sba {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
@@ -74,32 +81,46 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+inline namespace SBA_ELEM_NS {
+
+#ifdef SBA_ELEM_F16
+typedef _Float16 elem_t;
+#else
+typedef __bf16 elem_t;
+#endif
+typedef __attribute__((ext_vector_type(8))) elem_t el8;
+typedef __attribute__((ext_vector_type(2))) elem_t el2;
+
+__device__ __forceinline__ f32x16 mfma32(el8 a, el8 b, f32x16 c) {
+#ifdef SBA_ELEM_F16
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+#else
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+#endif
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
-// Round-to-nearest-even fp32 -> bf16 pairs (v_cvt_pk_bf16_f32 on gfx950).
-__device__ __forceinline__ bf16x2 cvt2(float a, float b) {
+// Round-to-nearest-even fp32 -> element pairs (v_cvt_pk_bf16_f32 / v_cvt_pk_f16_f32 on gfx950).
+__device__ __forceinline__ el2 cvt2(float a, float b) {
   f32x2 f = {a, b};
-  return __builtin_convertvector(f, bf16x2);
+  return __builtin_convertvector(f, el2);
 }
 
-__device__ __forceinline__ bf16x8 pack8(const float* p) {
-  bf16x2 a = cvt2(p[0], p[1]), b = cvt2(p[2], p[3]), c = cvt2(p[4], p[5]), d = cvt2(p[6], p[7]);
-  bf16x8 r;
+__device__ __forceinline__ el8 pack8(const float* p) {
+  el2 a = cvt2(p[0], p[1]), b = cvt2(p[2], p[3]), c = cvt2(p[4], p[5]), d = cvt2(p[6], p[7]);
+  el8 r;
   r[0] = a[0]; r[1] = a[1]; r[2] = b[0]; r[3] = b[1];
   r[4] = c[0]; r[5] = c[1]; r[6] = d[0]; r[7] = d[1];
   return r;
 }
 
-__device__ __forceinline__ bf16x8 zero8() {
-  bf16x8 r;
+__device__ __forceinline__ el8 zero8() {
+  el8 r;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) r[i] = (__bf16)0.0f;
+  for (int i = 0; i < 8; ++i) r[i] = (elem_t)0.0f;
   return r;
 }
 
@@ -123,14 +144,14 @@ __device__ __forceinline__ s16x4 lds_tr4(const unsigned short* p) {
 // MFMA operand (8 contraction slots per lane) gathered from a ROW-MAJOR LDS tile whose rows
 // are the contraction index.  `p0` / `p1` address rows 0..3 / 4..7 of the lane's 8-row group
 // as described for lds_tr4.
-__device__ __forceinline__ bf16x8 lds_tr8(const unsigned short* p0, const unsigned short* p1) {
+__device__ __forceinline__ el8 lds_tr8(const unsigned short* p0, const unsigned short* p1) {
   s16x4 a = lds_tr4(p0), b = lds_tr4(p1);
   s16x8 r = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
-  return __builtin_bit_cast(bf16x8, r);
+  return __builtin_bit_cast(el8, r);
 }
 
-__device__ __forceinline__ bf16x8 lds_row8(const unsigned short* p) {
-  return *reinterpret_cast<const bf16x8*>(p);
+__device__ __forceinline__ el8 lds_row8(const unsigned short* p) {
+  return *reinterpret_cast<const el8*>(p);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -302,15 +323,15 @@ __device__ __forceinline__ void stick_weights_fwd(const f32x16& x, float c, int 
 // ---------------------------------------------------------------------------------------------
 template <int D>
 __device__ __forceinline__ void store_block32(unsigned short* scratch, const f32x16 (&acc)[D / 32], float scale,
-                                              __bf16* out, int64_t stride_t, int row0, int limit, int lane) {
+                                              elem_t* out, int64_t stride_t, int row0, int limit, int lane) {
   const int n = lane & 31, h = lane >> 5;
-  __bf16* sc = reinterpret_cast<__bf16*>(scratch);
+  elem_t* sc = reinterpret_cast<elem_t*>(scratch);
 #pragma unroll
   for (int db = 0; db < D / 32; ++db) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int row = 8 * (i >> 2) + 4 * h + (i & 3);
-      sc[row * D + 32 * db + n] = (__bf16)(acc[db][i] * scale);
+      sc[row * D + 32 * db + n] = (elem_t)(acc[db][i] * scale);
     }
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own LDS writes have landed
@@ -331,16 +352,16 @@ __device__ __forceinline__ void store_block32(unsigned short* scratch, const f32
 // rounded again: one rounding fewer than a caller adding the two bf16 tensors afterwards.
 template <int D, class RowScale>
 __device__ __forceinline__ void store_block32_axpy(unsigned short* scratch, const f32x16 (&acc)[D / 32], float scale,
-                                                   __bf16* out, int64_t stride_t, int row0, int limit, int lane,
-                                                   const __bf16* addend, int64_t addend_stride_t, RowScale rowscale) {
+                                                   elem_t* out, int64_t stride_t, int row0, int limit, int lane,
+                                                   const elem_t* addend, int64_t addend_stride_t, RowScale rowscale) {
   const int n = lane & 31, h = lane >> 5;
-  __bf16* sc = reinterpret_cast<__bf16*>(scratch);
+  elem_t* sc = reinterpret_cast<elem_t*>(scratch);
 #pragma unroll
   for (int db = 0; db < D / 32; ++db) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int row = 8 * (i >> 2) + 4 * h + (i & 3);
-      sc[row * D + 32 * db + n] = (__bf16)(acc[db][i] * scale);
+      sc[row * D + 32 * db + n] = (elem_t)(acc[db][i] * scale);
     }
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own LDS writes have landed
@@ -351,15 +372,15 @@ __device__ __forceinline__ void store_block32_axpy(unsigned short* scratch, cons
     const int row = cidx / C8, c8 = cidx % C8;
     const bool ok = row0 + row < limit;
     const float f = rowscale(row);
-    const bf16x8 mine = *reinterpret_cast<const bf16x8*>(scratch + row * D + c8 * 8);
-    bf16x8 other;
+    const el8 mine = *reinterpret_cast<const el8*>(scratch + row * D + c8 * 8);
+    el8 other;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) other[e] = (__bf16)0.0f;
-    if (ok) other = *reinterpret_cast<const bf16x8*>(addend + (int64_t)(row0 + row) * addend_stride_t + c8 * 8);
+    for (int e = 0; e < 8; ++e) other[e] = (elem_t)0.0f;
+    if (ok) other = *reinterpret_cast<const el8*>(addend + (int64_t)(row0 + row) * addend_stride_t + c8 * 8);
     float sum[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) sum[e] = fmaf(f, (float)other[e], (float)mine[e]);
-    if (ok) *reinterpret_cast<bf16x8*>(out + (int64_t)(row0 + row) * stride_t + c8 * 8) = pack8(sum);
+    if (ok) *reinterpret_cast<el8*>(out + (int64_t)(row0 + row) * stride_t + c8 * 8) = pack8(sum);
   }
 }
 
@@ -386,10 +407,10 @@ struct Rows {
   unsigned row_bytes;   // stride between consecutive tokens, in bytes
 };
 
-__device__ __forceinline__ Rows make_rows(const __bf16* base, int64_t stride_t, int n_rows) {
+__device__ __forceinline__ Rows make_rows(const elem_t* base, int64_t stride_t, int n_rows) {
   Rows r;
   const uint64_t bytes = (uint64_t)n_rows * (uint64_t)stride_t * 2u;
-  r.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<__bf16*>(base), 0,
+  r.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<elem_t*>(base), 0,
                                              bytes > 0xffffffffull ? 0xffffffffu : (unsigned)bytes, 0x00020000);
   r.row_bytes = (unsigned)stride_t * 2u;
   return r;
@@ -400,8 +421,8 @@ __device__ __forceinline__ uint4 load16(const Rows& r, int row, int col_bytes) {
   return make_uint4(v[0], v[1], v[2], v[3]);
 }
 
-__device__ __forceinline__ bf16x8 load_frag(const Rows& r, int row, int col_bytes) {
-  return __builtin_bit_cast(bf16x8, load16(r, row, col_bytes));
+__device__ __forceinline__ el8 load_frag(const Rows& r, int row, int col_bytes) {
+  return __builtin_bit_cast(el8, load16(r, row, col_bytes));
 }
 
 // XOR swizzle of the 16-byte chunks of an UNPADDED row-major tile (row = D*2 bytes) that makes
@@ -475,4 +496,5 @@ __device__ __forceinline__ void wait_loads() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
+}  // inline namespace SBA_ELEM_NS
 }  // namespace sba

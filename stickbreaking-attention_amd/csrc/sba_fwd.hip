@@ -9,6 +9,7 @@
 #include <type_traits>
 
 namespace sba {
+inline namespace SBA_ELEM_NS {
 
 // WOUT: also write the attention weights (fp32, before their bf16 rounding) into a dense
 // [tokens x tokens] matrix per (batch, head) -- upstream's `return_attention` debug output
@@ -45,11 +46,11 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   const bool qvalid = qrow < t.doc_len;
 
   const int64_t tok0 = t.tok_start;
-  const __bf16* qb = reinterpret_cast<const __bf16*>(a.q.ptr) + t.batch * a.q.sb + head * a.q.sh + tok0 * a.q.st;
-  const __bf16* kb = reinterpret_cast<const __bf16*>(a.k.ptr) + t.batch * a.k.sb + head * a.k.sh + tok0 * a.k.st;
-  const __bf16* vb = reinterpret_cast<const __bf16*>(a.v.ptr) + t.batch * a.v.sb + head * a.v.sh + tok0 * a.v.st;
-  __bf16* ob = reinterpret_cast<__bf16*>(a.o.ptr) + t.batch * a.o.sb + head * a.o.sh + tok0 * a.o.st;
-  __bf16* rb = reinterpret_cast<__bf16*>(a.rem.ptr) + t.batch * a.rem.sb + head * a.rem.sh + tok0 * a.rem.st;
+  const elem_t* qb = reinterpret_cast<const elem_t*>(a.q.ptr) + t.batch * a.q.sb + head * a.q.sh + tok0 * a.q.st;
+  const elem_t* kb = reinterpret_cast<const elem_t*>(a.k.ptr) + t.batch * a.k.sb + head * a.k.sh + tok0 * a.k.st;
+  const elem_t* vb = reinterpret_cast<const elem_t*>(a.v.ptr) + t.batch * a.v.sb + head * a.v.sh + tok0 * a.v.st;
+  elem_t* ob = reinterpret_cast<elem_t*>(a.o.ptr) + t.batch * a.o.sb + head * a.o.sh + tok0 * a.o.st;
+  elem_t* rb = reinterpret_cast<elem_t*>(a.rem.ptr) + t.batch * a.rem.sb + head * a.rem.sh + tok0 * a.rem.st;
   const Rows qrows = make_rows(qb, a.q.st, t.doc_len);
   const Rows krows = make_rows(kb, a.k.st, t.doc_len);
   const Rows vrows = make_rows(vb, a.v.st, t.doc_len);
@@ -58,7 +59,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   const int kt_last = last_key / BF;
 
   // Q^T operand fragments: lane (n, h) holds Q[qrow][16*ks + 8*h .. +7] (zeros past the document).
-  bf16x8 qf[KS];
+  el8 qf[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) qf[ks] = load_frag(qrows, qrow, 32 * ks + 16 * h);
 
@@ -122,7 +123,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) x[i] = 0.0f;
     {
-      bf16x8 kfr[KS];
+      el8 kfr[KS];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) kfr[ks] = lds_row8(Kt + koff[ks]);
 #pragma unroll
@@ -150,7 +151,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
     }
     // P as the A operand of O = P.V: slot s of step tt is key 16*h + 8*tt + s, which the
     // permuted tile keeps in LDS row 16*tt + 8*(s/4) + 4*h + s%4.
-    bf16x8 vfr[2][DB];
+    el8 vfr[2][DB];
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
       const unsigned short* vrow = Vt + 16 * tt * D;
@@ -159,7 +160,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
     }
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
-      const bf16x8 pf = pack8(p + 8 * tt);
+      const el8 pf = pack8(p + 8 * tt);
 #pragma unroll
       for (int db = 0; db < DB; ++db) oacc[db] = mfma32(pf, vfr[tt][db], oacc[db]);
     }
@@ -177,7 +178,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   // epilogue: rem = what is left of the stick; o rows in the accumulator layout
   const float r = PROD ? carry : fast_exp2(carry);
   if (h == 0 && qvalid) {
-    rb[(int64_t)qrow * a.rem.st] = (__bf16)r;
+    rb[(int64_t)qrow * a.rem.st] = (elem_t)r;
     // rem in full precision for the backward of the fused output (last plane of the table)
     if (stick != nullptr) stick[(unsigned)(tab_rowplane32(t.doc_len) + qrow)] = r;
   }
@@ -231,4 +232,5 @@ hipError_t launch_fwd(const KArgs& a, int head_dim, bool ac, bool prod, bool wei
   return launch_fwd_d<64, false>(a, ac, prod, n_q_max, s);
 }
 
+}  // inline namespace SBA_ELEM_NS
 }  // namespace sba

@@ -42,15 +42,32 @@ struct ZeroArgs {
   const int* sched;
   int heads, tokens, head_dim;
   int64_t tab_stride;   // table entries per head available to the launch that wrote these outputs (< 0: no table in use)
+  unsigned nan_pair;    // two NaNs of the outputs' 16-bit element type
 };
 
 hipError_t launch_schedule(const SchedArgs& a, hipStream_t s);
 hipError_t launch_zero_tail(const ZeroArgs& a, hipStream_t s);
-hipError_t launch_fwd(const KArgs& a, int head_dim, bool attend_current, bool product, bool weights,
-                      int n_q_max, hipStream_t s);
-hipError_t launch_bwd_dq(const KArgs& a, int head_dim, bool attend_current, bool product, int n_q_max,
-                         hipStream_t s);
-hipError_t launch_bwd_dkdv(const KArgs& a, int head_dim, bool attend_current, bool product,
-                           int n_kv_max, hipStream_t s);
+
+// One set of compute launchers per element type (sba_fwd.hip and sba_bwd.hip are compiled once
+// for each, see SBA_ELEM_NS).
+#ifdef SBA_ELEM_F16
+#define SBA_INLINE_bf16
+#define SBA_INLINE_f16 inline
+#else
+#define SBA_INLINE_bf16 inline
+#define SBA_INLINE_f16
+#endif
+#define SBA_DECLARE_LAUNCHERS(NS)                                                                                \
+  SBA_INLINE_##NS namespace NS {                                                                                 \
+  hipError_t launch_fwd(const KArgs& a, int head_dim, bool attend_current, bool product, bool weights,           \
+                        int n_q_max, hipStream_t s);                                                             \
+  hipError_t launch_bwd_dq(const KArgs& a, int head_dim, bool attend_current, bool product, int n_q_max,         \
+                           hipStream_t s);                                                                       \
+  hipError_t launch_bwd_dkdv(const KArgs& a, int head_dim, bool attend_current, bool product, int n_kv_max,      \
+                             hipStream_t s);                                                                     \
+  }
+SBA_DECLARE_LAUNCHERS(bf16)
+SBA_DECLARE_LAUNCHERS(f16)
+#undef SBA_DECLARE_LAUNCHERS
 
 }  // namespace sba

@@ -195,7 +195,7 @@ __global__ void __launch_bounds__(256) zero_tail_kernel(const ZeroArgs a) {
   const int lo = max(row0, total), hi = min(row0 + ZERO_ROWS, a.tokens);
   if (lo >= hi) return;
   const int nrows = hi - lo, c8 = a.head_dim / 8;
-  const unsigned fill = refused ? 0x7fc07fc0u : 0u;   // two bf16 NaNs, or zeros
+  const unsigned fill = refused ? a.nan_pair : 0u;   // two NaNs of the element type, or zeros
   const uint4 z = make_uint4(fill, fill, fill, fill);
   for (int head = 0; head < a.heads; ++head) {
     for (int m = 0; m < a.n_mat; ++m) {

@@ -17,6 +17,7 @@ _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_PKG_DIR), "lib", "libsba.so")
 
 SBA_BF16 = 1
+SBA_F16 = 2
 FLAG_ATTEND_CURRENT = 1
 FLAG_CU_INT64 = 2
 FLAG_PRODUCT_SPACE = 4

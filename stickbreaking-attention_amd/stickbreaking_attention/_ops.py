@@ -158,22 +158,28 @@ _warned_dtypes = set()
 
 def _warn_reduced_precision(dtype) -> None:
     """Upstream runs its dots in the input dtype (tl.dot on fp16 / TF32 on fp32 inputs,
-    sb_varlen_fwd.py:42, utils.py:8); this library multiplies in bf16 whatever arrives.  Said once
-    per dtype instead of silently."""
+    sb_varlen_fwd.py:42, utils.py:8).  This library has kernels for bfloat16 and for float16 and
+    multiplies anything else in bfloat16.  Said once per dtype instead of silently."""
     if dtype not in _warned_dtypes:
         _warned_dtypes.add(dtype)
         warnings.warn(f"stickbreaking_attention: {dtype} inputs are rounded to bfloat16 before the matrix products "
                       "(8 bits of mantissa; outputs are returned in the input dtype)", stacklevel=4)
 
 
-def _prep(t: torch.Tensor, dpad: int, incoming_grad: bool = False) -> torch.Tensor:
-    """bf16, head_dim padded with zeros to `dpad`, row strides multiples of 8 elements (traceable).
-    The strides of an incoming gradient are not known while a backward is being traced, so
-    there it is simply made contiguous."""
-    if t.dtype != torch.bfloat16:
-        if not torch.compiler.is_compiling():
+def compute_dtype(dtype: torch.dtype) -> torch.dtype:
+    """The element type the kernels run in for inputs of `dtype`: bfloat16 and float16 natively (MFMA
+    of that type, fp32 accumulation), everything else in bfloat16."""
+    return dtype if dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
+
+
+def _prep(t: torch.Tensor, dpad: int, cdt: torch.dtype, incoming_grad: bool = False) -> torch.Tensor:
+    """Element type `cdt`, head_dim padded with zeros to `dpad`, row strides multiples of 8 elements
+    (traceable).  The strides of an incoming gradient are not known while a backward is being
+    traced, so there it is simply made contiguous."""
+    if t.dtype != cdt:
+        if not torch.compiler.is_compiling() and t.dtype not in (torch.bfloat16, torch.float16):
             _warn_reduced_precision(t.dtype)
-        t = t.to(torch.bfloat16)
+        t = t.to(cdt)
     d = t.shape[-1]
     if d != dpad:
         t = torch.nn.functional.pad(t, (0, dpad - d))
@@ -188,6 +194,10 @@ def _aligned(t: torch.Tensor) -> torch.Tensor:
     return t if t.data_ptr() % 16 == 0 else t.clone(memory_format=torch.contiguous_format)
 
 
+def _dtype_code(t: torch.Tensor) -> int:
+    return nat.SBA_F16 if t.dtype == torch.float16 else nat.SBA_BF16
+
+
 def _problem(q: torch.Tensor, fixed: bool, cu_seqlens: Optional[torch.Tensor], max_doc_len: int,
              inv_temp: float, attend_current: bool, product: bool, fused: bool):
     """The ``sba_problem`` of a launch plus the tensors whose pointers it holds."""
@@ -195,13 +205,13 @@ def _problem(q: torch.Tensor, fixed: bool, cu_seqlens: Optional[torch.Tensor], m
              (nat.FLAG_FUSE_REMAINDER if fused else 0))
     if fixed:
         B, H, T, d = q.shape
-        return nat.SbaProblem(nat.SBA_BF16, d, H, B, T, 0, T, flags | nat.FLAG_FIXED_LENGTH,
+        return nat.SbaProblem(_dtype_code(q), d, H, B, T, 0, T, flags | nat.FLAG_FIXED_LENGTH,
                               float(inv_temp), None), ()
     H, T, d = q.shape
     if cu_seqlens.dtype == torch.int64:
         flags |= nat.FLAG_CU_INT64
     cu = cu_seqlens.contiguous()
-    return nat.SbaProblem(nat.SBA_BF16, d, H, 1, T, cu.numel(), max_doc_len, flags, float(inv_temp),
+    return nat.SbaProblem(_dtype_code(q), d, H, 1, T, cu.numel(), max_doc_len, flags, float(inv_temp),
                           cu.data_ptr() if cu.numel() else None), (cu,)
 
 
@@ -316,7 +326,8 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
     d = q.shape[-1]
     dpad = _padded_dim(d)
     product = PRODUCT_SPACE
-    qp, kp, vp = (_prep(t, dpad) for t in (q, k, v))
+    cdt = compute_dtype(q.dtype)
+    qp, kp, vp = (_prep(t, dpad, cdt) for t in (q, k, v))
     lengths = None
     if fixed:
         B, H, T, _ = qp.shape
@@ -352,7 +363,7 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
                              bool(fused), o, rem, table, sched)
         if VALIDATE and not torch.compiler.is_compiling():
             check_status(sched, table, H)
-    if dpad != d or q.dtype != torch.bfloat16:
+    if dpad != d or q.dtype != cdt:
         o = o[..., :d].to(q.dtype)
         rem = rem.to(q.dtype)
     state = (table, sched, cu, max_len, product)
@@ -399,12 +410,13 @@ def run_backward(q, k, v, do, drem, fixed: bool, state, inv_temp: float, attend_
     table, sched, cu, max_len, product = state
     d = q.shape[-1]
     dpad = _padded_dim(d)
-    qp, kp, vp = (_prep(t, dpad) for t in (q, k, v))
-    dop = _prep(do, dpad, incoming_grad=True)
+    cdt = compute_dtype(q.dtype)
+    qp, kp, vp = (_prep(t, dpad, cdt) for t in (q, k, v))
+    dop = _prep(do, dpad, cdt, incoming_grad=True)
     if drem is None:
-        dremp = torch.empty(0, dtype=torch.bfloat16, device=q.device)
+        dremp = torch.empty(0, dtype=cdt, device=q.device)
     else:
-        dremp = drem if drem.dtype == torch.bfloat16 else drem.to(torch.bfloat16)
+        dremp = drem if drem.dtype == cdt else drem.to(cdt)
         if torch.compiler.is_compiling():
             dremp = dremp.contiguous()
     dq, dk, dv = torch.empty_like(qp), torch.empty_like(kp), torch.empty_like(vp)
@@ -415,7 +427,7 @@ def run_backward(q, k, v, do, drem, fixed: bool, state, inv_temp: float, attend_
     else:
         _compileable_backward(dop, dremp, qp, kp, vp, cu, max_len, float(inv_temp), bool(attend_current),
                               product, bool(fused), table, sched, gtab, dq, dk, dv)
-    if dpad != d or q.dtype != torch.bfloat16:
+    if dpad != d or q.dtype != cdt or k.dtype != cdt or v.dtype != cdt or dkdv_dtype not in (None, cdt):
         dq = dq[..., :d].to(q.dtype)
         dk = dk[..., :d].to(k.dtype if dkdv_dtype is None else dkdv_dtype)
         dv = dv[..., :d].to(v.dtype if dkdv_dtype is None else dkdv_dtype)

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for s in syms:
         assert hasattr(lib, s), f"{s} declared in include/sba.h but not exported"
     assert sorted(nat.EXPORTS) == syms
-    assert lib.sba_version() == 201
+    assert lib.sba_version() == 202
 
 
 def problem(**kw):
@@ -94,7 +94,7 @@ def test_undersized_workspaces_are_refused_on_the_host():
 
 
 @pytest.mark.parametrize("kw,code", [
-    (dict(head_dim=50), -2), (dict(dtype=7), -3), (dict(heads=0), -4), (dict(batch=2), -4),
+    (dict(head_dim=50), -2), (dict(dtype=7), -3), (dict(dtype=2, head_dim=50), -2), (dict(heads=0), -4), (dict(batch=2), -4),
     (dict(cu_seqlens=None), -1),
 ])
 def test_bad_problems_are_rejected_on_the_host(kw, code):

@@ -1,5 +1,5 @@
 """The edges of the supported input envelope: logits far outside N(0,1) in both carry spaces,
-genuinely fp32 inputs, and upstream's own long single-document case (tests/test_varlen.py:68-93:
+genuinely fp32 inputs, float16 inputs on the float16 kernels, and upstream's own long single-document case (tests/test_varlen.py:68-93:
 one 16384-token document, head_dim 128, shifted q/k that keep weight alive hundreds of keys
 from the diagonal)."""
 import os
@@ -79,6 +79,56 @@ def test_fp32_inputs_are_rounded_to_bf16_and_say_so():
     ref = orc.sb_varlen_grads(q, k, v, lengths, do)
     for name, gt, r in zip(("o", "rem", "dq", "dk", "dv"), (o.detach(), rem.detach(), dq, dk, dv), ref):
         assert_close(name + " (fp32 inputs)", gt, r)
+
+
+@pytest.mark.parametrize("d", [64, 128])
+def test_float16_runs_on_the_float16_kernels(d):
+    """float16 q, k, v, grad_o are multiplied as float16 (11 significant bits instead of bfloat16's 8;
+    upstream's tl.dot does the same, sb_varlen_fwd.py:42): the operands P and dZ and the outputs are
+    rounded eight times finer, so the error against the fp32 oracle on the same float16 values must
+    be several times below the bfloat16 gate.  No precision warning; float16 outputs; a refused
+    launch fills float16 NaNs."""
+    from stickbreaking_attention import _ops, sb_attn_varlen, sb_attn_varlen_fused
+    lengths = [300, 129, 64, 519]
+    T = sum(lengths)
+    g = torch.Generator().manual_seed(99 + d)
+    q, k, v, do = (torch.randn((3, T, d), generator=g).to(torch.float16) for _ in range(4))
+    assert not torch.equal(q, q.to(torch.bfloat16).to(torch.float16))      # not bf16-representable
+    ref = orc.sb_varlen_grads(q.float(), k.float(), v.float(), lengths, do.float())
+    for ac in (False, True):
+        with warnings.catch_warnings():
+            warnings.simplefilter("error")
+            got = _run(q, k, v, do, lengths, ac)
+        if ac:
+            ref = orc.sb_varlen_grads(q.float(), k.float(), v.float(), lengths, do.float(), None, True)
+        for name, gt, r in zip(("o", "rem", "dq", "dk", "dv"), got, ref):
+            assert gt.dtype == torch.float16
+            diff = (gt.float().cpu() - r).abs()
+            bound = 4e-3 + r.abs() * 2.0 ** -11
+            print(f"  {name} (float16, attend_current={ac}): max_abs={diff.max().item():.3e}")
+            assert (diff <= bound).all(), f"{name}: {diff.max().item():.3e}"
+    # fused output and its gradient
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    cu = cu_from_lengths(lengths, device=DEV)
+    out = sb_attn_varlen_fused(qg, kg, vg, cu, max(lengths), zero_start=False)
+    o_ref, rem_ref = orc.sb_varlen(q.float(), k.float(), v.float(), lengths)[:2]
+    fused_ref = o_ref + rem_ref[..., None] * v.float()
+    assert out.dtype == torch.float16
+    assert ((out.float().cpu() - fused_ref).abs() <= 4e-3 + fused_ref.abs() * 2.0 ** -11).all()
+
+
+def test_float16_refused_launch_gives_nan(monkeypatch):
+    from stickbreaking_attention import _ops
+    monkeypatch.setattr(_ops, "SYNC_FREE", True)
+    _ops.release_workspaces()
+    lengths = [700, 300]
+    g = torch.Generator().manual_seed(5)
+    q, k, v, do = (torch.randn((2, 1000, 64), generator=g).to(torch.float16) for _ in range(4))
+    from stickbreaking_attention import sb_attn_varlen
+    qg = q.to(DEV).requires_grad_()
+    o, rem = sb_attn_varlen(qg, k.to(DEV), v.to(DEV), cu_from_lengths(lengths, device=DEV), 64, zero_start=False)
+    torch.cuda.synchronize()
+    assert o.dtype == torch.float16 and torch.isnan(o).all() and torch.isnan(rem).all()
 
 
 def test_upstream_single_16k_document():

@@ -374,7 +374,7 @@ def test_other_head_dims_run_zero_padded(d):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
-def test_other_dtypes_are_computed_in_bf16(dtype):
+def test_other_dtypes_keep_their_dtype(dtype):
     from stickbreaking_attention import sb_attn
     q, k, v, do = orc.make_inputs((1, 2, 160, 64), 9, dist="upstream")   # bf16-representable values
     qg, kg, vg = (t.to(DEV).to(dtype).requires_grad_() for t in (q, k, v))
