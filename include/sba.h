@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define SBA_VERSION 202
+#define SBA_VERSION 203
 
 /* error codes (negative returns) */
 #define SBA_E_NULL      (-1)  /* a required pointer is NULL                         */
@@ -94,9 +94,11 @@ typedef struct sba_problem {
   int32_t  tokens;       /* T: tokens per batch entry (fixed) / total packed tokens      */
   int32_t  n_docs;       /* varlen: number of entries in cu_seqlens; fixed: ignored      */
   int32_t  max_doc_len;  /* upper bound on any document length (fixed: == tokens; 0 =
-                            unknown).  Only sba_table_bytes() looks at it; results never
-                            depend on it (upstream drops rows when its max_seqlens is
-                            too small, sb_varlen_fwd.py:478)                             */
+                            unknown, taken as `tokens`).  sba_table_bytes() sizes the
+                            tables with it and the backward its launches; the device
+                            checks it: a longer document makes the backward return
+                            at once with NaN outputs (upstream silently drops rows
+                            when its max_seqlens is too small, sb_varlen_fwd.py:478) */
   uint32_t flags;        /* SBA_ATTEND_CURRENT | SBA_CU_INT64 | SBA_PRODUCT_SPACE | ...  */
   float    inv_temp;     /* logit scale (upstream logit_scale / inv_temp)                */
   const void* cu_seqlens;/* varlen: inclusive cumulative document ends, WITHOUT a leading
@@ -130,7 +132,8 @@ size_t sba_table_bytes_for_lengths(const sba_problem* p, const int64_t* doc_leng
  * aligned and `schedule_size` (its size in bytes) at least sba_schedule_bytes(), else
  * SBA_E_WORKSPACE.  The first int32 of the workspace is a status word (0 = ok, else
  * SBA_STATUS_*) and the fourth the number of table entries per head the documents need, both
- * readable by the caller after the stream has drained.  Has no upstream counterpart as a
+ * readable by the caller after the stream has drained (the seventh: the longest document found).
+ * Has no upstream counterpart as a
  * separate call: upstream derives the tile of a program from its grid index inside `_forward`
  * (sb_varlen_fwd.py:281-296). */
 int sba_build_schedule(const sba_problem* p, void* schedule, size_t schedule_size, void* stream);
@@ -139,6 +142,8 @@ int sba_build_schedule(const sba_problem* p, void* schedule, size_t schedule_siz
 #define SBA_STATUS_BAD_CU           1   /* cu_seqlens not monotone or beyond `tokens`        */
 #define SBA_STATUS_TABLE_TOO_SMALL  4   /* reported by the Python layer when the fourth header
                                            word exceeds the entries per head of the tables   */
+#define SBA_STATUS_DOC_TOO_LONG     5   /* likewise when the seventh header word (the longest
+                                           document found) exceeds max_doc_len               */
 
 /* ---- forward ---------------------------------------------------------------------------- */
 
@@ -196,7 +201,7 @@ int sba_varlen_fwd_static(const sba_problem* p,
 /* ---- backward --------------------------------------------------------------------------- */
 
 /* dq, dk, dv for every token (zero for tokens that belong to no document; NaN everywhere when
- * nothing could run, as in the forward).  `schedule` and `stick_table` are the ones the forward
+ * nothing could run, as in the forward, or when a document is longer than max_doc_len).  `schedule` and `stick_table` are the ones the forward
  * of the same problem and inputs filled; `grad_table` is scratch; `table_size` is the size in
  * bytes of EACH of the two tables.  grad_rem may have ptr == NULL (treated as zeros). */
 int sba_varlen_bwd(const sba_problem* p, const void* schedule, size_t schedule_size,

@@ -2,6 +2,7 @@
 // in include/sba.h).  Host code only validates, sizes and launches.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <cstring>
 
@@ -178,6 +179,7 @@ int forward(const sba_problem* p, bool fixed, const void* schedule, size_t sched
   z.mat[0] = a.o; z.n_mat = 1; z.row = a.rem;
   z.sched = a.sched; z.heads = p->heads; z.tokens = p->tokens; z.head_dim = p->head_dim;
   z.tab_stride = a.tab_stride;
+  z.max_doc_len = -1;
   z.nan_pair = p->dtype == SBA_F16 ? 0x7e007e00u : 0x7fc07fc0u;
   return (int)launch_zero_tail(z, s);
 }
@@ -203,6 +205,15 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, size_t sche
   a.dq = to_view(dq); a.dk = to_view(dk); a.dv = to_view(dv);
   a.stick = const_cast<float*>(stick);
   a.gtab = gtab;
+  // Grid bounds of the dk/dv pass.  The second group of the key-tile list holds at most TAIL_TILES
+  // tiles of every document.  The first group holds ceil(L / BKV) - 1 tiles of a document of more
+  // than TAIL_TILES * BKV tokens and none of a shorter one: at most rows / BKV in all and, with the
+  // declared longest document, at most that many per document.  The declaration is checked on the
+  // device: a longer document makes every backward kernel return and the outputs NaN.
+  a.max_doc_len = (fixed || p->max_doc_len <= 0 || p->max_doc_len > p->tokens) ? p->tokens : p->max_doc_len;
+  const long long per_doc = (a.max_doc_len + BKV - 1) / BKV - kv_tail_tiles(a.max_doc_len);
+  const int n_long_max = (int)std::min<long long>(sz.rows / BKV, per_doc * sz.n_docs);
+  const int n_tail_max = (int)std::min<long long>(sz.n_kv_max, (long long)TAIL_TILES * sz.n_docs);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const bool ac = (p->flags & SBA_ATTEND_CURRENT) != 0, prod = (p->flags & SBA_PRODUCT_SPACE) != 0;
   hipError_t he = hipSuccess;
@@ -214,7 +225,7 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, size_t sche
     if (he != hipSuccess) return (int)he;
     {
       Timer tm(2, s);
-      he = (p->dtype == SBA_F16 ? f16::launch_bwd_dkdv : bf16::launch_bwd_dkdv)(a, p->head_dim, ac, prod, sz.n_kv_max, s);
+      he = (p->dtype == SBA_F16 ? f16::launch_bwd_dkdv : bf16::launch_bwd_dkdv)(a, p->head_dim, ac, prod, n_long_max, n_tail_max, s);
     }
   }
   if (he != hipSuccess || fixed) return (int)he;
@@ -223,6 +234,7 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, size_t sche
   z.mat[0] = a.dq; z.mat[1] = a.dk; z.mat[2] = a.dv; z.n_mat = 3;
   z.sched = a.sched; z.heads = p->heads; z.tokens = p->tokens; z.head_dim = p->head_dim;
   z.tab_stride = a.tab_stride;
+  z.max_doc_len = a.max_doc_len;
   z.nan_pair = p->dtype == SBA_F16 ? 0x7e007e00u : 0x7fc07fc0u;
   return (int)launch_zero_tail(z, s);
 }

@@ -15,6 +15,7 @@
 //                    the stick carry (table written by the forward) and the G prefix (table
 //                    written by bwd_dq_kernel) of each sub-block, recomputes p and dz and
 //                    accumulates dk and dv in registers; every output element is written once.
+//                    (bwd_dkdv_tail_kernel: the same for the key tiles that few queries follow.)
 //
 // Per-score math (upstream sb_varlen_bwd.py:439-453):
 //   G = A * (do.v - drem),  C = inclusive running sum of G over keys,  dz = G - beta * C,
@@ -119,7 +120,7 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, table entries needed
   const Tile t = reinterpret_cast<const Tile*>(sched + SCHED_HDR)[slot];
   asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch), "s"(t.tab_base));   // keep the tile read above the branch
-  if (hdr.x != 0 || slot >= hdr.y || hdr.w > a.tab_stride) return;
+  if (hdr.x != 0 || slot >= hdr.y || hdr.w > a.tab_stride || sched[SCHED_MAXLEN] > a.max_doc_len) return;
 
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -324,6 +325,9 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
 // step needs a single workgroup barrier and a tile has three steps to arrive.
 // -------------------------------------------------------------------------------------------
 constexpr int NT2 = 512;
+// Head dimensions for which the second group of key tiles (a handful of steps each, most of them on or
+// near the diagonal) goes to bwd_dkdv_tail_kernel instead.
+template <int D> struct TailKernel { static constexpr bool value = D == 64; };
 constexpr int BQ = 32;     // queries per step of the dk/dv pass
 constexpr int RING = 6;    // Q/dO tile slots: tiles i-1 (products) .. i+4 (in flight) of step i
 constexpr int AHEAD = 4;   // a tile is requested this many steps before the products use it + 1
@@ -349,7 +353,10 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, table entries needed
   const Tile t = reinterpret_cast<const Tile*>(sched + a.kv_list_off)[slot];
   asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch), "s"(t.tab_base));   // keep the tile read above the branch
-  if (hdr.x != 0 || slot >= hdr.z || hdr.w > a.tab_stride) return;
+  // with a kernel of their own for the documents' last key tiles, this one stops where they begin
+  const int2 hdr2 = *reinterpret_cast<const int2*>(sched + SCHED_MAXLEN);   // longest document, key tiles of the first group
+  const int n_mine = TailKernel<D>::value ? hdr2.y : hdr.z;
+  if (hdr.x != 0 || slot >= n_mine || hdr.w > a.tab_stride || hdr2.x > a.max_doc_len) return;
   const int kt = t.idx;
 
   const int tid = threadIdx.x;
@@ -725,6 +732,192 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   }
 }
 
+// -------------------------------------------------------------------------------------------
+// dk / dv of the second group of key tiles (kv_tail_tiles): at most TAIL_TILES * BKV queries see such a
+// tile.  For packed short documents that is the whole dk/dv pass, and the eight-wave pipeline
+// above spends nearly all of such a tile on its prologue, its barriers and its epilogue with one
+// workgroup per CU.  Here a workgroup is four independent waves: wave w owns the 32 keys of block
+// w, recomputes p and dz of the query blocks at or after it exactly as a score wave does, turns
+// its own 32x32 blocks around through a private piece of LDS and accumulates its own rows of dk
+// and dv.  One barrier (after the Q / dO rows have landed), two workgroups per CU.
+// -------------------------------------------------------------------------------------------
+template <int D, bool AC, bool PROD>
+__global__ void __launch_bounds__(NT, 2) bwd_dkdv_tail_kernel(const KArgs a) {
+  constexpr int KS = D / 16, DB = D / 32;
+  constexpr int QROWS = TAIL_TILES * BKV;            // queries that can follow the tile's first key
+  __shared__ __attribute__((aligned(16))) unsigned short Qs[QROWS * D];   // Q rows from the tile's first key on (swizzled like every tile)
+  __shared__ __attribute__((aligned(16))) unsigned short Gs[QROWS * D];   // dO rows
+  __shared__ __attribute__((aligned(16))) unsigned short St[NT / 64][2][32 * 32];   // per wave: p and dz of one block, [query][key]
+
+  const int* sched = a.sched;
+  const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, table entries needed
+  const int2 hdr2 = *reinterpret_cast<const int2*>(sched + SCHED_MAXLEN);   // longest document, key tiles of the first group
+  if (hdr.x != 0 || hdr.w > a.tab_stride || hdr2.x > a.max_doc_len) return;
+  const int which = blockIdx.x / a.heads;
+  const int head = blockIdx.x - which * a.heads;
+  const int slot = hdr2.y + which;
+  if (slot >= hdr.z) return;
+  const Tile t = reinterpret_cast<const Tile*>(sched + a.kv_list_off)[slot];
+  const int kt = t.idx;
+  const int L = t.doc_len;
+
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63, n = lane & 31, h = lane >> 5;
+  const int i16 = lane & 15, blk = (lane >> 4) & 1;
+
+  const int64_t tok0 = t.tok_start;
+  const elem_t* qb = reinterpret_cast<const elem_t*>(a.q.ptr) + t.batch * a.q.sb + head * a.q.sh + tok0 * a.q.st;
+  const elem_t* kb = reinterpret_cast<const elem_t*>(a.k.ptr) + t.batch * a.k.sb + head * a.k.sh + tok0 * a.k.st;
+  const elem_t* vb = reinterpret_cast<const elem_t*>(a.v.ptr) + t.batch * a.v.sb + head * a.v.sh + tok0 * a.v.st;
+  const elem_t* gob = reinterpret_cast<const elem_t*>(a.go.ptr) + t.batch * a.go.sb + head * a.go.sh + tok0 * a.go.st;
+  const Rows qrows = make_rows(qb, a.q.st, L);
+  const Rows grows = make_rows(gob, a.go.st, L);
+  const Rows krows = make_rows(kb, a.k.st, L);
+  const Rows vrows = make_rows(vb, a.v.st, L);
+
+  const int q_first = kt * BKV;                      // first query that can see the tile
+  const int nblk = (L - q_first + 31) / 32;          // 1 .. QROWS / 32 query blocks
+  // all of those Q and dO rows at once (rows past the document arrive as zeros)
+  {
+    TileCopy<D, QROWS, NT, false> qcopy, gcopy;
+    qcopy.init(tid, qrows.row_bytes);
+    gcopy.init(tid, grows.row_bytes);
+    qcopy.issue(qrows, q_first, Qs, 32 * nblk);      // (32 rows per instruction: whole query blocks)
+    gcopy.issue(grows, q_first, Gs, 32 * nblk);
+  }
+  // Wave w of workgroup b takes key block (w + b) mod 4: the block with the most queries behind it
+  // is the first one, and two workgroups that share a CU should not both put it on the same SIMD.
+  const int kblk = (w + blockIdx.x) & (BKV / 32 - 1);
+  const int k0 = q_first + 32 * kblk;                // this wave's keys
+  const bool active = k0 < L;
+  el8 kf[KS], vf[KS];                                // MFMA row n holds key k0 + kperm(n)
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    kf[ks] = load_frag(krows, k0 + kperm(n), 32 * ks + 16 * h);
+    vf[ks] = load_frag(vrows, k0 + kperm(n), 32 * ks + 16 * h);
+  }
+  // A block that starts past the end of the document is never visible; its table reads are
+  // redirected into the document's area and never used.
+  const int tblock = min((BKV / 32) * kt + kblk, (L - 1) / 32);
+  const int64_t tab_row0 = (int64_t)head * a.tab_stride + t.tab_base;
+  const int64_t tab = tab_row0 + tab_seg32(L, tblock);
+  const int64_t tab_rowval = tab_row0 + tab_rowplane32(L);
+  struct Raw { float e, g, d; };
+  auto request = [&](int qblk, Raw& r) {             // the carries of a query block, clamped into the document
+    const int qrow = q_first + 32 * qblk + n;
+    const int qc = qrow < L ? qrow : L - 1;
+    r.e = a.stick[tab + qc];
+    r.g = a.gtab[tab + qc];
+    r.d = a.gtab[tab_rowval + qc];
+  };
+  Raw cur, nxt;
+  request(kblk, cur);
+  float rem_own = 0.0f;       // fused output: rem_j * do_j reaches dv_j through the diagonal of P (see above)
+  if (a.fuse && k0 + n < L) rem_own = a.stick[tab_rowval + k0 + n];
+
+  int roff[KS], xoff[2], yoff[2][DB];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) roff[ks] = swz_off<D>(n, 2 * ks + h);
+  // The private p / dz blocks have rows of 64 bytes (4 chunks).  A transpose read takes 4 whole
+  // consecutive rows, which are 256 contiguous bytes whatever the order of the chunks inside a row;
+  // the 16-byte row writes of 16 lanes are spread over the banks by rotating the chunks with row/4.
+  auto blk_off = [](int row, int chunk) { return row * 32 + ((chunk ^ ((row >> 2) & 3)) << 3); };
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int r = 8 * h + 4 * u + (i16 >> 2);
+    const int xc = 16 * blk + 4 * (i16 & 3);                    // key column inside the block (elements)
+    xoff[u] = blk_off(r, xc >> 3) + (xc & 7);
+#pragma unroll
+    for (int j = 0; j < DB; ++j) {
+      const int yc = 32 * j + 16 * blk + 4 * (i16 & 3);         // d column (elements)
+      yoff[u][j] = swz_off<D>(r, yc >> 3) + (yc & 7);
+    }
+  }
+  f32x16 acc_v[DB], acc_k[DB];
+#pragma unroll
+  for (int j = 0; j < DB; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { acc_v[j][i] = 0.0f; acc_k[j][i] = 0.0f; }
+
+  wait_loads<0>();
+  lds_barrier();              // the only barrier: every wave's part of the Q / dO rows has landed
+  if (!active) return;
+
+  unsigned short* Pt = St[w][0];
+  unsigned short* Zt = St[w][1];
+  // query blocks at or after the key block (those before it see none of these keys)
+#pragma unroll 1
+  for (int qblk = kblk; qblk < nblk; ++qblk) {
+    request(qblk + 1, nxt);                           // (clamped; unused past the last block)
+    const int qw0 = q_first + 32 * qblk;
+    const int qrow = qw0 + n;
+    const bool ok = qrow < L;
+    float carry_e = ok ? cur.e : (PROD ? 1.0f : 0.0f);
+    float carry_c = ok ? cur.g : 0.0f;
+    const float dr = ok ? cur.d : 0.0f;
+    f32x16 x, da;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) { x[j] = 0.0f; da[j] = 0.0f; }
+    {
+      const unsigned short* Qt = Qs + 32 * qblk * D;
+      const unsigned short* Gt = Gs + 32 * qblk * D;
+      el8 qfr[KS], gfr[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) { qfr[ks] = lds_row8(Qt + roff[ks]); gfr[ks] = lds_row8(Gt + roff[ks]); }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        x = mfma32(kf[ks], qfr[ks], x);
+        da = mfma32(vf[ks], gfr[ks], da);
+      }
+    }
+    el8 pf[2], zf[2];
+    {
+      float p[16], bt[16], ends[2] = {0.0f, 0.0f};
+      grad_weights<AC, PROD>(x, a.c, k0, qw0, qrow, h, carry_e, p, bt, ends);
+      if (a.fuse && qblk == kblk) {
+        float pd[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) pd[j] = p[j] + (16 * h + j == n ? rem_own : 0.0f);
+        pf[0] = pack8(pd);
+        pf[1] = pack8(pd + 8);
+      } else {
+        pf[0] = pack8(p);
+        pf[1] = pack8(p + 8);
+      }
+      grad_dz<PROD>(p, bt, da, ends, h, carry_c, dr, zf);
+    }
+    // turn the block around: [query][key] rows in, key-major MFMA operands out
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      *reinterpret_cast<el8*>(Pt + blk_off(n, 2 * h + tt)) = pf[tt];
+      *reinterpret_cast<el8*>(Zt + blk_off(n, 2 * h + tt)) = zf[tt];
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own writes have landed
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const el8 ap = lds_tr8(Pt + xoff[0] + 16 * ks * 32, Pt + xoff[1] + 16 * ks * 32);
+      const el8 az = lds_tr8(Zt + xoff[0] + 16 * ks * 32, Zt + xoff[1] + 16 * ks * 32);
+      const unsigned short* Gr = Gs + (32 * qblk + 16 * ks) * D;
+      const unsigned short* Qr = Qs + (32 * qblk + 16 * ks) * D;
+#pragma unroll
+      for (int j = 0; j < DB; ++j) {
+        acc_v[j] = mfma32(ap, lds_tr8(Gr + yoff[0][j], Gr + yoff[1][j]), acc_v[j]);
+        acc_k[j] = mfma32(az, lds_tr8(Qr + yoff[0][j], Qr + yoff[1][j]), acc_k[j]);
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the reads are done before the next block overwrites the piece
+    cur = nxt;
+  }
+  // the private piece becomes the output scratch (32 x D elements: exactly its size)
+  static_assert(2 * 32 * 32 == 32 * D, "the staging piece of a wave doubles as its output scratch");
+  elem_t* dvb = reinterpret_cast<elem_t*>(a.dv.ptr) + t.batch * a.dv.sb + head * a.dv.sh + tok0 * a.dv.st;
+  elem_t* dkb = reinterpret_cast<elem_t*>(a.dk.ptr) + t.batch * a.dk.sb + head * a.dk.sh + tok0 * a.dk.st;
+  store_block32<D>(Pt, acc_v, 1.0f, dvb, a.dv.st, k0, L, lane);
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  store_block32<D>(Pt, acc_k, a.inv_temp, dkb, a.dk.st, k0, L, lane);
+}
+
 // Explicit instantiations: every (head_dim, attend_current, carry space) variant the launchers use.
 template __global__ void bwd_dq_kernel<64, false, false>(const KArgs);
 template __global__ void bwd_dq_kernel<64, false, true>(const KArgs);
@@ -734,6 +927,10 @@ template __global__ void bwd_dq_kernel<128, false, false>(const KArgs);
 template __global__ void bwd_dq_kernel<128, false, true>(const KArgs);
 template __global__ void bwd_dq_kernel<128, true, false>(const KArgs);
 template __global__ void bwd_dq_kernel<128, true, true>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<64, false, false>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<64, false, true>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<64, true, false>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<64, true, true>(const KArgs);
 template __global__ void bwd_dkdv_kernel<64, false, false>(const KArgs);
 template __global__ void bwd_dkdv_kernel<64, false, true>(const KArgs);
 template __global__ void bwd_dkdv_kernel<64, true, false>(const KArgs);
@@ -756,15 +953,32 @@ static hipError_t launch_dq_d(const KArgs& a, bool ac, bool prod, int n_q_max, h
   return hipGetLastError();
 }
 
+// n_long_max / n_last_max: upper bounds on the key tiles of the first / second group of the list.
 template <int D>
-static hipError_t launch_dkdv_d(const KArgs& a, bool ac, bool prod, int n_kv_max, hipStream_t s) {
-  const dim3 grid((unsigned)n_kv_max * (unsigned)a.heads), block(NT2);
-  if (ac) {
-    if (prod) hipLaunchKernelGGL((bwd_dkdv_kernel<D, true, true>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((bwd_dkdv_kernel<D, true, false>), grid, block, 0, s, a);
-  } else {
-    if (prod) hipLaunchKernelGGL((bwd_dkdv_kernel<D, false, true>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((bwd_dkdv_kernel<D, false, false>), grid, block, 0, s, a);
+static hipError_t launch_dkdv_d(const KArgs& a, bool ac, bool prod, int n_long_max, int n_last_max, hipStream_t s) {
+  const bool split = TailKernel<D>::value;
+  const unsigned n_main = split ? (unsigned)n_long_max : (unsigned)(n_long_max + n_last_max);
+  if (n_main > 0) {
+    const dim3 grid(n_main * (unsigned)a.heads), block(NT2);
+    if (ac) {
+      if (prod) hipLaunchKernelGGL((bwd_dkdv_kernel<D, true, true>), grid, block, 0, s, a);
+      else hipLaunchKernelGGL((bwd_dkdv_kernel<D, true, false>), grid, block, 0, s, a);
+    } else {
+      if (prod) hipLaunchKernelGGL((bwd_dkdv_kernel<D, false, true>), grid, block, 0, s, a);
+      else hipLaunchKernelGGL((bwd_dkdv_kernel<D, false, false>), grid, block, 0, s, a);
+    }
+  }
+  if constexpr (TailKernel<D>::value) {
+    if (n_last_max > 0) {
+      const dim3 grid((unsigned)n_last_max * (unsigned)a.heads), block(NT);
+      if (ac) {
+        if (prod) hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, true, true>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, true, false>), grid, block, 0, s, a);
+      } else {
+        if (prod) hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, false, true>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, false, false>), grid, block, 0, s, a);
+      }
+    }
   }
   return hipGetLastError();
 }
@@ -774,9 +988,10 @@ hipError_t launch_bwd_dq(const KArgs& a, int head_dim, bool ac, bool prod, int n
   return launch_dq_d<64>(a, ac, prod, n_q_max, s);
 }
 
-hipError_t launch_bwd_dkdv(const KArgs& a, int head_dim, bool ac, bool prod, int n_kv_max, hipStream_t s) {
-  if (head_dim == 128) return launch_dkdv_d<128>(a, ac, prod, n_kv_max, s);
-  return launch_dkdv_d<64>(a, ac, prod, n_kv_max, s);
+hipError_t launch_bwd_dkdv(const KArgs& a, int head_dim, bool ac, bool prod, int n_long_max, int n_last_max,
+                           hipStream_t s) {
+  if (head_dim == 128) return launch_dkdv_d<128>(a, ac, prod, n_long_max, n_last_max, s);
+  return launch_dkdv_d<64>(a, ac, prod, n_long_max, n_last_max, s);
 }
 
 }  // inline namespace SBA_ELEM_NS

@@ -32,6 +32,14 @@ constexpr int BM = 128;  // query rows per workgroup tile (4 waves x 32 rows)
 constexpr int BN = 64;   // keys per KV tile staged in LDS by the dq pass
 constexpr int BKV = 128;  // keys owned by one workgroup of the dk/dv pass
 constexpr int BT = 32;   // keys per carry-table entry (one MFMA sub-block)
+// The key-tile list has two groups.  The second holds the tiles that few queries follow, for which
+// the dk/dv pass has a lighter kernel: every tile of a document of at most TAIL_TILES * BKV tokens,
+// and the last tile of every longer document.  The first group holds the rest.
+constexpr int TAIL_TILES = 2;
+__host__ __device__ inline int kv_tail_tiles(int len) {   // key tiles of a document in the second group
+  const int nkv = (len + BKV - 1) / BKV;
+  return len <= TAIL_TILES * BKV ? nkv : 1;
+}
 constexpr int NT = 256;  // threads per workgroup
 
 // Schedule workspace layout (int32 words).
@@ -40,7 +48,8 @@ constexpr int SCHED_NQ = 1;      // number of query tiles
 constexpr int SCHED_NKV = 2;     // number of KV tiles
 constexpr int SCHED_TABLE = 3;   // carry-table entries per head the documents need (saturates at INT_MAX)
 constexpr int SCHED_TOTAL = 4;   // tokens covered by the documents (0 when the input is rejected)
-constexpr int SCHED_MAXLEN = 5;  // longest document found
+constexpr int SCHED_MAXLEN = 6;  // longest document found (read together with the next word: keep the pair 8-byte aligned)
+constexpr int SCHED_NKV_LONG = 7; // key tiles of the first group of the key-tile list (see kv_tail_tiles)
 constexpr int SCHED_HDR = 16;    // tile lists start here
 constexpr int TILE_WORDS = 8;    // int32 words of one Tile
 
@@ -478,9 +487,12 @@ struct TileCopy {
     voff = src * (int)row_bytes + logical * 16;
   }
 
-  __device__ __forceinline__ void issue(const Rows& r, int row0, unsigned short* lds_tile) const {
+  // `rows_needed` (uniform): instructions whose rows all lie at or beyond it are skipped; the tile
+  // rows they would have filled keep whatever they held.
+  __device__ __forceinline__ void issue(const Rows& r, int row0, unsigned short* lds_tile, int rows_needed = ROWS) const {
 #pragma unroll
     for (int j = 0; j < NCH; ++j) {
+      if (!KEYS && j * STEP >= rows_needed) continue;
       const int soff = __builtin_amdgcn_readfirstlane((row0 + row_delta(j)) * (int)r.row_bytes);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           r.rsrc, (__attribute__((address_space(3))) void*)(lds_tile + (j * STEP + wave * RPI) * D), 16,

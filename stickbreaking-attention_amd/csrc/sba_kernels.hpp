@@ -21,6 +21,8 @@ struct KArgs {
   int tokens;                  // tokens per batch entry
   int fuse;                    // the output is o + rem * v (and grad_o is the gradient of that)
   int64_t tab_stride;          // carry-table entries per head the caller's tables hold
+  int max_doc_len;             // backward: the longest document the caller declared (its grids are sized with it;
+                               // the kernels refuse to run when the scheduler found a longer one)
   float c;                     // inv_temp * log2(e)
   float inv_temp;
 };
@@ -43,6 +45,7 @@ struct ZeroArgs {
   int heads, tokens, head_dim;
   int64_t tab_stride;   // table entries per head available to the launch that wrote these outputs (< 0: no table in use)
   unsigned nan_pair;    // two NaNs of the outputs' 16-bit element type
+  int max_doc_len;      // longest document the launch was sized for (< 0: the launch does not depend on it)
 };
 
 hipError_t launch_schedule(const SchedArgs& a, hipStream_t s);
@@ -63,8 +66,8 @@ hipError_t launch_zero_tail(const ZeroArgs& a, hipStream_t s);
                         int n_q_max, hipStream_t s);                                                             \
   hipError_t launch_bwd_dq(const KArgs& a, int head_dim, bool attend_current, bool product, int n_q_max,         \
                            hipStream_t s);                                                                       \
-  hipError_t launch_bwd_dkdv(const KArgs& a, int head_dim, bool attend_current, bool product, int n_kv_max,      \
-                             hipStream_t s);                                                                     \
+  hipError_t launch_bwd_dkdv(const KArgs& a, int head_dim, bool attend_current, bool product, int n_long_max,    \
+                             int n_last_max, hipStream_t s);                                                     \
   }
 SBA_DECLARE_LAUNCHERS(bf16)
 SBA_DECLARE_LAUNCHERS(f16)

@@ -27,6 +27,7 @@ FLAG_FUSE_REMAINDER = 16
 STATUS_MESSAGES = {
     1: "cu_seqlens is not a non-decreasing sequence within [0, total_tokens]",
     4: "the carry tables are too small for the documents in cu_seqlens (max_seqlens under-states a document)",
+    5: "a document in cu_seqlens is longer than max_seqlens (the backward refuses to run: its outputs are NaN)",
 }
 
 

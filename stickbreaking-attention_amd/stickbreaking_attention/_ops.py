@@ -362,7 +362,7 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
         _compileable_forward(qp, kp, vp, cu, max_len, float(inv_temp), bool(attend_current), product,
                              bool(fused), o, rem, table, sched)
         if VALIDATE and not torch.compiler.is_compiling():
-            check_status(sched, table, H)
+            check_status(sched, table, H, max_len)
     if dpad != d or q.dtype != cdt:
         o = o[..., :d].to(q.dtype)
         rem = rem.to(q.dtype)
@@ -370,13 +370,17 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
     return (o, rem, state, weights) if return_attention else (o, rem, state)
 
 
-def check_status(sched: torch.Tensor, table: Optional[torch.Tensor] = None, heads: int = 1) -> None:
-    """Read the scheduler's status words back (synchronises) and raise on malformed cu_seqlens or on
-    carry tables smaller than the documents need."""
-    hdr = sched[:16].view(torch.int32).tolist()
-    status, need = hdr[0], hdr[3]
-    if status == 0 and table is not None and table.numel() and need > table.numel() // heads:
+def check_status(sched: torch.Tensor, table: Optional[torch.Tensor] = None, heads: int = 1,
+                 max_doc_len: Optional[int] = None) -> None:
+    """Read the scheduler's status words back (synchronises) and raise on malformed cu_seqlens, on
+    carry tables smaller than the documents need, or on a document longer than the declared
+    ``max_doc_len`` (which the backward's launch is sized with)."""
+    hdr = sched[:32].view(torch.int32).tolist()
+    status, need, longest = hdr[0], hdr[3], hdr[6]
+    if status == 0 and table is not None and table.numel() and need > ((table.numel() // heads) & ~31):
         status = 4
+    if status == 0 and max_doc_len is not None and longest > max_doc_len:
+        status = 5
     if status != 0:
         raise ValueError("sb_attn_varlen: " + nat.STATUS_MESSAGES.get(status, f"scheduler status {status}"))
 

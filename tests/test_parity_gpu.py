@@ -152,6 +152,31 @@ def test_understated_max_seqlens(monkeypatch):
         run_varlen(q, k, v, do, lengths, max_seqlens=64)
 
 
+def test_understated_max_seqlens_with_roomy_tables(monkeypatch):
+    """Without the lengths on the host the backward's launches are sized with max_seqlens.  A
+    document longer than declared whose tables still fit (many short documents leave room) is seen
+    by the device: the forward, which does not depend on the bound, is right; the backward
+    returns NaN, and validation names the reason."""
+    from stickbreaking_attention import _ops, sb_attn_varlen
+    monkeypatch.setattr(_ops, "SYNC_FREE", True)
+    _ops.release_workspaces()
+    lengths = [300] + [20] * 60
+    T = sum(lengths)
+    q, k, v, do = orc.make_inputs((2, T, 64), 78)
+    ref = oracle_varlen(q, k, v, do, lengths)
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    cu = cu_from_lengths(lengths, device=DEV)
+    o, rem = sb_attn_varlen(qg, kg, vg, cu, 256, zero_start=False)          # 300 > 256
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do.to(DEV))
+    torch.cuda.synchronize()
+    check_all((o.detach(), rem.detach()), ref[:2])
+    for t in (dq, dk, dv):
+        assert torch.isnan(t).all()
+    monkeypatch.setattr(_ops, "VALIDATE", True)
+    with pytest.raises(ValueError, match="longer than max_seqlens"):
+        sb_attn_varlen(qg, kg, vg, cu, 256, zero_start=False)
+
+
 def test_no_documents_give_zero_outputs():
     from stickbreaking_attention import sb_attn_varlen
     q = torch.randn(2, 128, 64, device=DEV).to(torch.bfloat16).requires_grad_()
