@@ -10,12 +10,14 @@
 
 namespace sba {
 
-constexpr int SCHED_THREADS = 1024;
 constexpr int RANK_LIMIT = 4096;   // beyond this many documents the input order is kept
 
 __device__ __forceinline__ int cdiv(int a, int b) { return (a + b - 1) / b; }
 
 // Scratch (int32) behind the two tile lists, per document: start, len, order, qoff, kvoff, table base.
+// SCHED_THREADS: workgroup size; a small one when there are few documents (every step of the scans
+// and every phase boundary is a workgroup barrier, which costs by the wave).
+template <int SCHED_THREADS>
 __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a) {
   __shared__ int s_status, s_maxlen;
   __shared__ int s_scan_q[SCHED_THREADS], s_scan_kv[SCHED_THREADS], s_scan_ne[SCHED_THREADS];
@@ -26,6 +28,7 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
   // be three quarters of this kernel's time.  Beyond RANK_LIMIT documents the same arrays in the
   // workspace are used.
   __shared__ int s_len[RANK_LIMIT], s_ord[RANK_LIMIT], s_qoff[RANK_LIMIT + 1], s_kvoff[RANK_LIMIT + 1];
+  __shared__ int s_start[RANK_LIMIT], s_tab[RANK_LIMIT];
   const int tid = threadIdx.x;
   const int nd = a.n_docs;
   int* hdr = a.out;
@@ -43,6 +46,8 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
   int* const ranked = in_lds ? s_ord : order;         // rank -> document index
   int* const q_before = in_lds ? s_qoff : qoff;       // by rank: query tiles of the documents ranked before
   int* const kv_before = in_lds ? s_kvoff : kvoff;    // by rank: key tiles of the first group ranked before
+  int* const start_of = in_lds ? s_start : dstart;    // by document index: first token
+  int* const tab_of = in_lds ? s_tab : dtab;          // by document index: first carry-table entry
 
   if (tid == 0) { s_status = 0; s_maxlen = 0; }
   __syncthreads();
@@ -67,6 +72,7 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
       len = (int)(en - st);
     }
     dstart[d] = (int)st;
+    if (in_lds) s_start[d] = (int)st;
     dlen[d] = len;
     if (in_lds) s_len[d] = len;
     atomicMax(&s_maxlen, len);
@@ -135,12 +141,12 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
       const int d = ranked[i];
       const int len = len_of[d];
       q_before[i] = bq; kv_before[i] = bkv;
-      dtab[d] = tab_ok ? (int)btab : 0;
+      tab_of[d] = tab_ok ? (int)btab : 0;
       if (ok) {              // the document's last key tiles, in the second group (the older one first: more steps)
         const int nkv = cdiv(len, BKV), ntail = kv_tail_tiles(len);
         for (int j2 = 0; j2 < ntail; ++j2) {
           Tile t;
-          t.tok_start = fixed ? 0 : dstart[d];
+          t.tok_start = fixed ? 0 : start_of[d];
           t.doc_len = len;
           t.idx = nkv - ntail + j2;
           t.batch = fixed ? d : 0;
@@ -179,11 +185,11 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
     }
     const int nq = cdiv(len_of[d], BM);
     Tile t;
-    t.tok_start = fixed ? 0 : dstart[d];
+    t.tok_start = fixed ? 0 : start_of[d];
     t.doc_len = len_of[d];
     t.idx = nq - 1 - within;             // newest (most expensive) query tile first
     t.batch = fixed ? d : 0;
-    t.tab_base = dtab[d];
+    t.tab_base = tab_of[d];
     t.rsv[0] = t.rsv[1] = t.rsv[2] = 0;
     qtiles[s] = t;
   }
@@ -195,11 +201,11 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
     while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (kv_before[mid] <= s) lo = mid; else hi = mid; }
     const int d = ranked[lo];
     Tile t;
-    t.tok_start = fixed ? 0 : dstart[d];
+    t.tok_start = fixed ? 0 : start_of[d];
     t.doc_len = len_of[d];
     t.idx = s - kv_before[lo];               // oldest keys are seen by the most queries: first
     t.batch = fixed ? d : 0;
-    t.tab_base = dtab[d];
+    t.tab_base = tab_of[d];
     t.rsv[0] = t.rsv[1] = t.rsv[2] = 0;
     kvtiles[s] = t;
   }
@@ -246,7 +252,8 @@ __global__ void __launch_bounds__(256) zero_tail_kernel(const ZeroArgs a) {
 }
 
 hipError_t launch_schedule(const SchedArgs& a, hipStream_t s) {
-  hipLaunchKernelGGL(sched_kernel, dim3(1), dim3(SCHED_THREADS), 0, s, a);
+  if (a.n_docs <= 512) hipLaunchKernelGGL(sched_kernel<256>, dim3(1), dim3(256), 0, s, a);
+  else hipLaunchKernelGGL(sched_kernel<1024>, dim3(1), dim3(1024), 0, s, a);
   return hipGetLastError();
 }
 
