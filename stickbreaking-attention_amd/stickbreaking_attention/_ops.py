@@ -14,6 +14,7 @@ while ``torch.compile`` traces.  The registered operators return nothing and wri
 buffers the caller allocated, so they need no shape function.
 """
 import ctypes
+import functools
 import math
 import os
 import warnings
@@ -75,8 +76,9 @@ def workspace_sizes(fixed: bool, batch: int, heads: int, tokens: int, n_docs: in
                     lengths: Optional[Sequence[int]] = None) -> Tuple[int, int]:
     """(schedule bytes, floats of one carry table): the same numbers as ``sba_schedule_bytes`` and
     ``sba_table_bytes // 4`` (``sba_table_bytes_for_lengths // 4`` when the document lengths are
-    given), computed without touching the library so that they can be evaluated while a graph is
-    being traced (checked against the library in the tests)."""
+    given -- or, as an int, the table entries per head they were already found to need), computed
+    without touching the library so that they can be evaluated while a graph is being traced
+    (checked against the library in the tests)."""
     docs = batch if fixed else n_docs
     rows = (batch if fixed else 1) * tokens
     n_q = rows // _BM + docs + 1
@@ -85,7 +87,7 @@ def workspace_sizes(fixed: bool, batch: int, heads: int, tokens: int, n_docs: in
     if fixed:
         entries = batch * table_entries(tokens)
     elif lengths is not None:
-        entries = max(32, sum(table_entries(int(n)) for n in lengths))
+        entries = lengths if isinstance(lengths, int) else max(32, sum(table_entries(int(n)) for n in lengths))
     else:
         entries = table_entries_bound(tokens, max_doc_len, n_docs)
     return (4 * words + 255) & ~255, heads * entries
@@ -138,7 +140,7 @@ def remember_host_cu(cu_seqlens: torch.Tensor, vals: Sequence[int]) -> None:
     if version is None or torch.compiler.is_compiling():
         return
     _host_cu_cache[:] = [e for e in _host_cu_cache if e[0]() is not None][-(_HOST_CU_CACHE_SIZE - 1):]
-    _host_cu_cache.append((weakref.ref(cu_seqlens), version, tuple(int(x) for x in vals)))
+    _host_cu_cache.append((weakref.ref(cu_seqlens), version, vals if isinstance(vals, tuple) else tuple(int(x) for x in vals)))
 
 
 def _doc_lengths(cu_vals: Sequence[int], tokens: int) -> Tuple[int, ...]:
@@ -151,6 +153,14 @@ def _doc_lengths(cu_vals: Sequence[int], tokens: int) -> Tuple[int, ...]:
         out.append(end - prev)
         prev = end
     return tuple(out)
+
+
+@functools.lru_cache(maxsize=16)
+def _lengths_info(cu_vals: Tuple[int, ...], tokens: int) -> Tuple[Tuple[int, ...], int, int]:
+    """(document lengths, longest document (at least 1), carry-table entries per head) of a cu_seqlens
+    whose values are on the host; remembered, because a model calls every layer with the same one."""
+    lengths = _doc_lengths(cu_vals, tokens)
+    return lengths, max(1, max(lengths, default=1)), max(32, sum(table_entries(n) for n in lengths))
 
 
 _warned_dtypes = set()
@@ -342,8 +352,7 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
         if cu_vals is not None:
             # lengths known on the host: malformed input raises here, the tables get their exact
             # size, and results do not depend on max_seqlens at all
-            lengths = _doc_lengths(cu_vals, T)
-            max_len = max(1, max(lengths, default=1))
+            _, max_len, lengths = _lengths_info(cu_vals, T)     # (`lengths`: the table entries they need)
     sched_bytes, table_floats = workspace_sizes(fixed, B, H, T, n_docs, max_len, lengths)
     # Every row is written by the library: rows of documents by the forward kernel, rows that
     # belong to no document are cleared (upstream leaves those uninitialised).
