@@ -201,6 +201,25 @@ def test_empty_documents_and_tail_tokens():
 
 
 @pytest.mark.parametrize("ac", [False, True])
+@pytest.mark.parametrize("d", [64, 128])
+def test_key_tile_group_boundaries(d, ac, monkeypatch):
+    """Document lengths on both sides of every boundary of the dk/dv pass's tile grouping (all key
+    tiles of a document of up to 256 tokens and the last tile of a longer one go to the four-wave
+    kernel at head_dim 64): 1, 32, 33, 128, 129, 255, 256, 257, 384, 385 tokens, with a gradient
+    for rem as well, once with the lengths on the host and once with launches sized from the bound."""
+    from stickbreaking_attention import _ops
+    lengths = [257, 1, 128, 385, 33, 256, 129, 32, 384, 255]
+    T = sum(lengths)
+    q, k, v, do = orc.make_inputs((2, T, d), 4242 + d)
+    drem = torch.randn((2, T), generator=torch.Generator().manual_seed(7)).to(torch.bfloat16)
+    ref = oracle_varlen(q, k, v, do, lengths, ac, drem=drem)
+    check_all(run_varlen(q, k, v, do, lengths, ac, drem=drem), ref)
+    monkeypatch.setattr(_ops, "SYNC_FREE", True)
+    _ops.release_workspaces()
+    check_all(run_varlen(q, k, v, do, lengths, ac, drem=drem, max_seqlens=400), ref)
+
+
+@pytest.mark.parametrize("ac", [False, True])
 @pytest.mark.parametrize("H,L", [(3, 4096), (12, 4096), (3, 8192)])
 def test_upstream_varlen_grid(H, L, ac):
     """The upstream test's own shapes and input distribution (single long document, d=128,
