@@ -166,22 +166,16 @@ int forward(const sba_problem* p, bool fixed, const void* schedule, size_t sched
   a.q = to_view(q); a.k = to_view(k); a.v = to_view(v); a.o = to_view(o); a.rem = to_view(rem);
   a.stick = stick;
   a.weights = weights;
+  a.clear_spare = fixed ? 0 : 1;
+  a.nan_pair = p->dtype == SBA_F16 ? 0x7e007e00u : 0x7fc07fc0u;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   hipError_t he = hipSuccess;
-  if (sz.n_docs > 0) {
+  {   // (packed input without a single document still launches: the spare workgroups clear the outputs)
     Timer tm(0, s, timed);
     he = (p->dtype == SBA_F16 ? f16::launch_fwd : bf16::launch_fwd)(a, p->head_dim, (p->flags & SBA_ATTEND_CURRENT) != 0,
                     (p->flags & SBA_PRODUCT_SPACE) != 0, weights != nullptr, sz.n_q_max, s);
   }
-  if (he != hipSuccess || fixed) return (int)he;
-  ZeroArgs z;
-  std::memset(&z, 0, sizeof(z));
-  z.mat[0] = a.o; z.n_mat = 1; z.row = a.rem;
-  z.sched = a.sched; z.heads = p->heads; z.tokens = p->tokens; z.head_dim = p->head_dim;
-  z.tab_stride = a.tab_stride;
-  z.max_doc_len = -1;
-  z.nan_pair = p->dtype == SBA_F16 ? 0x7e007e00u : 0x7fc07fc0u;
-  return (int)launch_zero_tail(z, s);
+  return (int)he;
 }
 
 int backward(const sba_problem* p, bool fixed, const void* schedule, size_t sched_bytes, const sba_view* q,
@@ -216,27 +210,18 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, size_t sche
   const int n_tail_max = (int)std::min<long long>(sz.n_kv_max, (long long)TAIL_TILES * sz.n_docs);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const bool ac = (p->flags & SBA_ATTEND_CURRENT) != 0, prod = (p->flags & SBA_PRODUCT_SPACE) != 0;
+  a.clear_spare = fixed ? 0 : 1;
+  a.nan_pair = p->dtype == SBA_F16 ? 0x7e007e00u : 0x7fc07fc0u;
   hipError_t he = hipSuccess;
-  if (sz.n_docs > 0) {
-    {
-      Timer tm(1, s);
-      he = (p->dtype == SBA_F16 ? f16::launch_bwd_dq : bf16::launch_bwd_dq)(a, p->head_dim, ac, prod, sz.n_q_max, s);
-    }
-    if (he != hipSuccess) return (int)he;
-    {
-      Timer tm(2, s);
-      he = (p->dtype == SBA_F16 ? f16::launch_bwd_dkdv : bf16::launch_bwd_dkdv)(a, p->head_dim, ac, prod, n_long_max, n_tail_max, s);
-    }
+  {
+    Timer tm(1, s);
+    he = (p->dtype == SBA_F16 ? f16::launch_bwd_dq : bf16::launch_bwd_dq)(a, p->head_dim, ac, prod, sz.n_q_max, s);
   }
-  if (he != hipSuccess || fixed) return (int)he;
-  ZeroArgs z;
-  std::memset(&z, 0, sizeof(z));
-  z.mat[0] = a.dq; z.mat[1] = a.dk; z.mat[2] = a.dv; z.n_mat = 3;
-  z.sched = a.sched; z.heads = p->heads; z.tokens = p->tokens; z.head_dim = p->head_dim;
-  z.tab_stride = a.tab_stride;
-  z.max_doc_len = a.max_doc_len;
-  z.nan_pair = p->dtype == SBA_F16 ? 0x7e007e00u : 0x7fc07fc0u;
-  return (int)launch_zero_tail(z, s);
+  if (he == hipSuccess && sz.n_docs > 0) {
+    Timer tm(2, s);
+    he = (p->dtype == SBA_F16 ? f16::launch_bwd_dkdv : bf16::launch_bwd_dkdv)(a, p->head_dim, ac, prod, n_long_max, n_tail_max, s);
+  }
+  return (int)he;
 }
 
 // Schedule workspace of sba_varlen_fwd_static: one array per GPU, inside the code object, so the

@@ -120,7 +120,18 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, table entries needed
   const Tile t = reinterpret_cast<const Tile*>(sched + SCHED_HDR)[slot];
   asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch), "s"(t.tab_base));   // keep the tile read above the branch
-  if (hdr.x != 0 || slot >= hdr.y || hdr.w > a.tab_stride || sched[SCHED_MAXLEN] > a.max_doc_len) return;
+  const bool refused = hdr.x != 0 || hdr.w > a.tab_stride || sched[SCHED_MAXLEN] > a.max_doc_len;
+  if (refused || slot >= hdr.y) {
+    if (a.clear_spare) {     // for the dk/dv pass as well, which has no slots to spare
+      int row0, row1;
+      unsigned pair;
+      spare_rows(refused, slot, hdr.y, sched[SCHED_TOTAL], a.tokens, a.nan_pair, row0, row1, pair);
+      fill_rows16(a.dq, head, row0, row1, D, pair, threadIdx.x, NT);
+      fill_rows16(a.dk, head, row0, row1, D, pair, threadIdx.x, NT);
+      fill_rows16(a.dv, head, row0, row1, D, pair, threadIdx.x, NT);
+    }
+    return;
+  }
 
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);

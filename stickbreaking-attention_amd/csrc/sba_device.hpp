@@ -82,6 +82,40 @@ struct View {
   int64_t sb, sh, st;  // element strides
 };
 
+// Fills rows [row0, row1) of one head of a [heads, tokens, width] 16-bit tensor (width a multiple of
+// 8 elements, rows 16-byte aligned) or of a per-row tensor (width 1) with a repeated 16-bit value.
+__device__ inline void fill_rows16(const View& v, int head, int row0, int row1, int width, unsigned pair,
+                                   int tid, int nthreads) {
+  if (v.ptr == nullptr || row1 <= row0) return;
+  unsigned short* base = reinterpret_cast<unsigned short*>(v.ptr) + head * v.sh;
+  if (width == 1) {
+    for (int r = row0 + tid; r < row1; r += nthreads) base[(int64_t)r * v.st] = (unsigned short)pair;
+    return;
+  }
+  const int c8 = width / 8;
+  const uint4 z = make_uint4(pair, pair, pair, pair);
+  for (int i = tid; i < (row1 - row0) * c8; i += nthreads) {
+    const int r = row0 + i / c8, c = i % c8;
+    *reinterpret_cast<uint4*>(base + (int64_t)r * v.st + c * 8) = z;
+  }
+}
+
+// Upstream leaves the rows of `o`, `dq`, `dk`, `dv` past cu_seqlens[-1] uninitialised (empty_like,
+// sb_varlen_fwd.py:418) and relies on zeros_like elsewhere (sb_varlen_bwd.py:507-509).  Here the
+// compute kernels write every row of every document exactly once, and the workgroups a launch has
+// to spare clear the rest: the grid of a query-tile-owned kernel has one slot per 128 tokens more
+// than the documents can use, so slot (tiles + j) takes the j-th block of 128 rows behind the last
+// document.  When nothing else runs -- the scheduler rejected cu_seqlens, the carry tables are
+// smaller than the documents need, a document is longer than declared -- every slot fills its
+// own 128 rows of the token axis with NaN instead, so that the failure cannot pass for a result.
+// Returns the rows this workgroup has to fill: [row0, row1), and with what.
+__device__ inline void spare_rows(bool refused, int slot, int n_tiles, int total, int tokens, unsigned nan_pair,
+                                  int& row0, int& row1, unsigned& pair) {
+  row0 = refused ? slot * BM : total + (slot - n_tiles) * BM;
+  row1 = min(row0 + BM, tokens);
+  pair = refused ? nan_pair : 0u;
+}
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains every
 // outstanding GLOBAL load (s_waitcnt vmcnt(0)), which would expose the full latency of the
 // tile prefetches and table reads that are deliberately kept in flight across the barrier.

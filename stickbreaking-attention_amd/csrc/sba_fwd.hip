@@ -35,7 +35,17 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, table entries needed
   const Tile t = reinterpret_cast<const Tile*>(sched + SCHED_HDR)[slot];
   asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch));   // keep the tile read above the branch
-  if (hdr.x != 0 || slot >= hdr.y || (a.stick != nullptr && hdr.w > a.tab_stride)) return;
+  const bool refused = hdr.x != 0 || (a.stick != nullptr && hdr.w > a.tab_stride);
+  if (refused || slot >= hdr.y) {
+    if (a.clear_spare) {
+      int row0, row1;
+      unsigned pair;
+      spare_rows(refused, slot, hdr.y, sched[SCHED_TOTAL], a.tokens, a.nan_pair, row0, row1, pair);
+      fill_rows16(a.o, head, row0, row1, D, pair, threadIdx.x, NT);
+      fill_rows16(a.rem, head, row0, row1, 1, pair, threadIdx.x, NT);
+    }
+    return;
+  }
 
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);

@@ -20,6 +20,9 @@ struct KArgs {
   int heads;
   int tokens;                  // tokens per batch entry
   int fuse;                    // the output is o + rem * v (and grad_o is the gradient of that)
+  int clear_spare;             // packed input: spare workgroups clear the rows that belong to no document (or fill
+                               // everything with NaN when the launch is refused)
+  unsigned nan_pair;           // two NaNs of the 16-bit element type
   int64_t tab_stride;          // carry-table entries per head the caller's tables hold
   int max_doc_len;             // backward: the longest document the caller declared (its grids are sized with it;
                                // the kernels refuse to run when the scheduler found a longer one)
@@ -36,20 +39,7 @@ struct SchedArgs {
   int* out;
 };
 
-// Rows of packed variable-length outputs that belong to no document.
-struct ZeroArgs {
-  View mat[3];      // [heads, tokens, head_dim] outputs to clear past the last document
-  int n_mat;
-  View row;         // per-row output (rem); ptr may be null
-  const int* sched;
-  int heads, tokens, head_dim;
-  int64_t tab_stride;   // table entries per head available to the launch that wrote these outputs (< 0: no table in use)
-  unsigned nan_pair;    // two NaNs of the outputs' 16-bit element type
-  int max_doc_len;      // longest document the launch was sized for (< 0: the launch does not depend on it)
-};
-
 hipError_t launch_schedule(const SchedArgs& a, hipStream_t s);
-hipError_t launch_zero_tail(const ZeroArgs& a, hipStream_t s);
 
 // One set of compute launchers per element type (sba_fwd.hip and sba_bwd.hip are compiled once
 // for each, see SBA_ELEM_NS).

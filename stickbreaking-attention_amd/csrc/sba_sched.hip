@@ -220,46 +220,9 @@ __global__ void __launch_bounds__(SCHED_THREADS) sched_kernel(const SchedArgs a)
   }
 }
 
-// Upstream leaves the rows of `o`, `dq`, `dk`, `dv` past cu_seqlens[-1] uninitialised
-// (empty_like, sb_varlen_fwd.py:418) and relies on zeros_like elsewhere (sb_varlen_bwd.py:507-509).
-// Here the compute kernels write every row of every document exactly once, so only the rows
-// that belong to no document need clearing: 64 rows per workgroup, which exits at once when
-// its rows are covered.  When nothing else ran -- the scheduler rejected cu_seqlens, or the
-// carry tables handed in are smaller than the documents need -- every row is filled with NaN
-// instead, so that the failure cannot pass for a result.
-constexpr int ZERO_ROWS = 64;
-__global__ void __launch_bounds__(256) zero_tail_kernel(const ZeroArgs a) {
-  const bool refused = a.sched[SCHED_STATUS] != 0 || (a.tab_stride >= 0 && a.sched[SCHED_TABLE] > a.tab_stride) ||
-                       (a.max_doc_len >= 0 && a.sched[SCHED_MAXLEN] > a.max_doc_len);
-  const int total = refused ? 0 : a.sched[SCHED_TOTAL];
-  const int row0 = blockIdx.x * ZERO_ROWS;
-  const int lo = max(row0, total), hi = min(row0 + ZERO_ROWS, a.tokens);
-  if (lo >= hi) return;
-  const int nrows = hi - lo, c8 = a.head_dim / 8;
-  const unsigned fill = refused ? a.nan_pair : 0u;   // two NaNs of the element type, or zeros
-  const uint4 z = make_uint4(fill, fill, fill, fill);
-  for (int head = 0; head < a.heads; ++head) {
-    for (int m = 0; m < a.n_mat; ++m) {
-      unsigned short* base = reinterpret_cast<unsigned short*>(a.mat[m].ptr) + head * a.mat[m].sh + lo * a.mat[m].st;
-      for (int c = threadIdx.x; c < nrows * c8; c += 256)
-        *reinterpret_cast<uint4*>(base + (c / c8) * a.mat[m].st + (c % c8) * 8) = z;
-    }
-    if (a.row.ptr != nullptr) {
-      unsigned short* base = reinterpret_cast<unsigned short*>(a.row.ptr) + head * a.row.sh + lo * a.row.st;
-      for (int r = threadIdx.x; r < nrows; r += 256) base[r * a.row.st] = (unsigned short)fill;
-    }
-  }
-}
-
 hipError_t launch_schedule(const SchedArgs& a, hipStream_t s) {
   if (a.n_docs <= 512) hipLaunchKernelGGL(sched_kernel<256>, dim3(1), dim3(256), 0, s, a);
   else hipLaunchKernelGGL(sched_kernel<1024>, dim3(1), dim3(1024), 0, s, a);
-  return hipGetLastError();
-}
-
-hipError_t launch_zero_tail(const ZeroArgs& a, hipStream_t s) {
-  if (a.tokens <= 0) return hipSuccess;
-  hipLaunchKernelGGL(zero_tail_kernel, dim3((a.tokens + ZERO_ROWS - 1) / ZERO_ROWS), dim3(256), 0, s, a);
   return hipGetLastError();
 }
 
