@@ -189,7 +189,7 @@ int sba_attn_fwd_weights(const sba_problem* p, const void* schedule, size_t sche
  * schedule workspace is a fixed array of SBA_STATIC_SCRATCH_BYTES bytes that lives inside the
  * library's code object on every GPU it runs on, from the first call until the process ends; the
  * call allocates and frees nothing.  Problems whose sba_schedule_bytes() exceed that size are
- * rejected with SBA_E_WORKSPACE (the array holds, for example, 262144 tokens in 8192 documents).
+ * rejected with SBA_E_WORKSPACE (the array holds, for example, 262144 tokens in 4096 documents).
  * All calls on one GPU share that GPU's array: calls that overlap on one GPU (different streams
  * or threads) race; serialise them.  The first call on a device looks the array's address up
  * (hipGetSymbolAddress): make that call outside any graph capture. */
