@@ -157,6 +157,16 @@ def measure(name, steps, warmup, args, torch, lib, lengths_override=None):
         with torch.no_grad():
             return attention()
 
+    # An idle MI355X sits at a few hundred MHz and takes some tenths of a second of load to reach
+    # its working clock; a handful of warm-up steps (10 ms) ends long before that.  The same step is
+    # therefore repeated, untimed, for `ramp_ms` before the W warm-up steps and the K timed steps.
+    t0 = time.perf_counter()
+    ramp_steps = 0
+    while (time.perf_counter() - t0) * 1e3 < args.ramp_ms:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+        ramp_steps += 10
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -178,11 +188,11 @@ def measure(name, steps, warmup, args, torch, lib, lengths_override=None):
     # per-kernel durations: HIP events recorded by the library on the stream it launches on
     lib.sba_set_timing(1)
     acc = [0.0, 0.0, 0.0]
-    reps = 5
+    reps = 10
     for _ in range(reps):
         step()
         for i in range(3):
-            acc[i] += lib.sba_last_kernel_ms(i)
+            acc[i] += lib.sba_last_kernel_ms(i)   # waits for that kernel of the step just queued
     lib.sba_set_timing(0)
     kern_ms = [a / reps for a in acc]
     if not backward:
@@ -193,7 +203,7 @@ def measure(name, steps, warmup, args, torch, lib, lengths_override=None):
     del q, k, v, do
     torch.cuda.empty_cache()
     return dict(name=name, lengths=lengths, cfg=cfg, H=H, d=d, T=T, fixed=fixed, backward=backward, pairs=pairs,
-                tensor_bytes=tensor_bytes, ms_step=ms_step, ms_fwd=ms_fwd, kern_ms=kern_ms)
+                tensor_bytes=tensor_bytes, ms_step=ms_step, ms_fwd=ms_fwd, kern_ms=kern_ms, ramp_steps=ramp_steps)
 
 
 def roofline(m, lib):
@@ -232,6 +242,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--ramp-ms", type=float, default=400.0,
+                    help="untimed repetitions of the step before the warm-up, until the device clock has settled")
     ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
     ap.add_argument("--lengths", default=None,
                     help="comma-separated document lengths replacing the workload's own (shape sweeps; "
@@ -278,6 +290,7 @@ def main():
         "value": total_flops / (m["ms_step"] * 1e-3) / 1e12,
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": m["ms_step"],
+        "clock_ramp": {"ms": args.ramp_ms, "untimed_steps_before_warmup": m["ramp_steps"]},
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": describe(m).replace(m["name"] + ":", label + ":", 1),

@@ -224,12 +224,13 @@ int         sba_version(void);
 const char* sba_error_string(int code);
 
 /* Benchmark instrumentation, NOT part of the re-entrant interface: with the switch on, every
- * compute launch is bracketed by HIP events on the caller's stream and the call WAITS for the
- * kernel (host synchronisation, event creation); sba_last_kernel_ms returns the duration in
- * milliseconds of the most recent launch of each kernel (which: 0 = forward, 1 = backward dq pass,
- * 2 = backward dk/dv pass).  One process-wide switch and one process-wide set of results (the
- * backward may run on PyTorch's autograd thread): do not use with concurrent callers, under
- * graph capture, or in production.  Off by default; sba_varlen_fwd_static ignores it. */
+ * compute launch is bracketed by HIP events on the caller's stream (event creation, no waiting:
+ * timed kernels follow one another on the device as untimed ones do); sba_last_kernel_ms WAITS
+ * for the most recent launch of the kernel asked for and returns its duration in milliseconds
+ * (which: 0 = forward, 1 = backward dq pass, 2 = backward dk/dv pass).  One process-wide switch
+ * and one process-wide set of results (the backward may run on PyTorch's autograd thread): do
+ * not use with concurrent callers, under graph capture, or in production.  Off by default;
+ * sba_varlen_fwd_static ignores it. */
 void  sba_set_timing(int on);
 float sba_last_kernel_ms(int which);
 

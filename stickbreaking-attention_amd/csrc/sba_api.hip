@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <atomic>
 #include <cstring>
+#include <mutex>
 
 #include "sba.h"
 #include "sba_kernels.hpp"
@@ -100,26 +101,36 @@ int check_arch() {
   return cached ? 0 : SBA_E_ARCH;
 }
 
-struct Timer {
+// Brackets one compute launch with HIP events on the caller's stream.  Nothing waits here: the
+// pair is parked and resolved when sba_last_kernel_ms asks for it, so that timed kernels follow
+// one another on the device exactly as untimed ones do.
+struct EventPair {
   hipEvent_t e0 = nullptr, e1 = nullptr;
+};
+std::mutex g_ev_mutex;
+EventPair g_ev[3];
+
+struct Timer {
+  EventPair ev;
   hipStream_t s;
   int which;
   bool on;
   Timer(int which_, hipStream_t s_, bool allowed = true) : s(s_), which(which_), on(allowed && g_timing.load() != 0) {
     if (on) {
-      on = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess;
-      if (on) (void)hipEventRecord(e0, s);
+      on = hipEventCreate(&ev.e0) == hipSuccess && hipEventCreate(&ev.e1) == hipSuccess;
+      if (on) (void)hipEventRecord(ev.e0, s);
     }
   }
   ~Timer() {
+    EventPair done = ev;   // (timing off, or creation failed half-way: nothing to park)
     if (on) {
-      (void)hipEventRecord(e1, s);
-      (void)hipEventSynchronize(e1);
-      float ms = 0.f;
-      if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess) g_ms[which].store(ms);
+      (void)hipEventRecord(ev.e1, s);
+      std::lock_guard<std::mutex> lock(g_ev_mutex);
+      done = g_ev[which];
+      g_ev[which] = ev;
     }
-    if (e0) (void)hipEventDestroy(e0);
-    if (e1) (void)hipEventDestroy(e1);
+    if (done.e0) (void)hipEventDestroy(done.e0);
+    if (done.e1) (void)hipEventDestroy(done.e1);
   }
 };
 
@@ -379,6 +390,15 @@ int sba_varlen_fwd_static(const sba_problem* p, const sba_view* q, const sba_vie
 }
 
 void sba_set_timing(int on) { g_timing.store(on); }
-float sba_last_kernel_ms(int which) { return (which >= 0 && which < 3) ? g_ms[which].load() : 0.f; }
+float sba_last_kernel_ms(int which) {
+  if (which < 0 || which >= 3) return 0.f;
+  std::lock_guard<std::mutex> lock(g_ev_mutex);
+  const EventPair& ev = g_ev[which];
+  float ms = 0.f;
+  if (ev.e0 != nullptr && ev.e1 != nullptr && hipEventSynchronize(ev.e1) == hipSuccess &&
+      hipEventElapsedTime(&ms, ev.e0, ev.e1) == hipSuccess)
+    g_ms[which].store(ms);
+  return g_ms[which].load();
+}
 
 }  // extern "C"
