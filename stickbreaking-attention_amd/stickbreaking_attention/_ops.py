@@ -98,6 +98,11 @@ _host_cu_cache = []
 _HOST_CU_CACHE_SIZE = 8
 
 
+# views without the leading zero that sb_attn_varlen already handed out:
+# (weak reference to cu_seqlens, version, view), newest last
+_stripped_views = []
+
+
 def _version_of(t):
     """The in-place modification counter of a tensor, or None where PyTorch keeps none (tensors
     created under ``torch.inference_mode()`` raise on ``_version``)."""
@@ -237,7 +242,7 @@ def _nbytes(t: Optional[torch.Tensor]) -> int:
 
 
 def _launch_fwd(fixed: bool, q, k, v, cu_seqlens, max_doc_len: int, logit_scale: float, attend_current: bool,
-                product: bool, fused: bool, o, rem, table, sched, weights=None) -> None:
+                product: bool, fused: bool, o, rem, table, sched, weights=None, build_schedule: bool = True) -> None:
     nat.require_gpu(q)
     lib = nat.load()
     q, k, v = _aligned(q), _aligned(k), _aligned(v)
@@ -248,7 +253,8 @@ def _launch_fwd(fixed: bool, q, k, v, cu_seqlens, max_doc_len: int, logit_scale:
     with torch.cuda.device(q.device):
         stream = nat.stream_ptr(q.device)
         # every workspace goes in with its size: the library answers SBA_E_WORKSPACE instead of overrunning one
-        nat.check(lib.sba_build_schedule(ctypes.byref(prob), sched.data_ptr(), _nbytes(sched), stream), "sba_build_schedule")
+        if build_schedule:
+            nat.check(lib.sba_build_schedule(ctypes.byref(prob), sched.data_ptr(), _nbytes(sched), stream), "sba_build_schedule")
         code = fn(ctypes.byref(prob), sched.data_ptr(), _nbytes(sched),
                   ctypes.byref(nat.view4(q, fixed)), ctypes.byref(nat.view4(k, fixed)),
                   ctypes.byref(nat.view4(v, fixed)), ctypes.byref(nat.view4(o, fixed)),
@@ -282,9 +288,10 @@ def _launch_bwd(fixed: bool, do, dr, q, k, v, cu_seqlens, max_doc_len: int, logi
 @custom_op("varlen_fwd", mutates_args={"o", "rem", "table", "sched"})
 def _compileable_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens: torch.Tensor,
                          max_seqlens: int, logit_scale: float, attend_current: bool, product: bool, fused: bool,
-                         o: torch.Tensor, rem: torch.Tensor, table: torch.Tensor, sched: torch.Tensor) -> None:
+                         o: torch.Tensor, rem: torch.Tensor, table: torch.Tensor, sched: torch.Tensor,
+                         build_schedule: bool = True) -> None:
     _launch_fwd(False, q, k, v, cu_seqlens, max_seqlens, logit_scale, attend_current, product, fused,
-                o, rem, table, sched)
+                o, rem, table, sched, build_schedule=build_schedule)
 
 
 @custom_op("varlen_bwd", mutates_args={"gtab", "dq", "dk", "dv"})
@@ -299,8 +306,9 @@ def _compileable_backward(do: torch.Tensor, dr: torch.Tensor, q: torch.Tensor, k
 @custom_op("attn_fwd", mutates_args={"o", "rem", "table", "sched"})
 def _compileable_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_scale: float, attend_current: bool,
                      product: bool, fused: bool, o: torch.Tensor, rem: torch.Tensor, table: torch.Tensor,
-                     sched: torch.Tensor) -> None:
-    _launch_fwd(True, q, k, v, None, q.shape[2], logit_scale, attend_current, product, fused, o, rem, table, sched)
+                     sched: torch.Tensor, build_schedule: bool = True) -> None:
+    _launch_fwd(True, q, k, v, None, q.shape[2], logit_scale, attend_current, product, fused, o, rem, table, sched,
+                build_schedule=build_schedule)
 
 
 @custom_op("attn_bwd", mutates_args={"gtab", "dq", "dk", "dv"})
@@ -323,6 +331,37 @@ def _check_cu(cu_seqlens: torch.Tensor, like: torch.Tensor) -> torch.Tensor:
     if cu_seqlens.device != like.device:
         cu_seqlens = cu_seqlens.to(like.device)
     return cu_seqlens
+
+
+# Schedules already built on a device: the tile lists depend only on the documents (cu_seqlens, or
+# batch and length of a fixed-length call) and on the token count, and a model hands the same
+# cu_seqlens tensor to every layer, so the scheduler kernel runs once per tensor instead of once per
+# layer.  Entries: (weak reference to cu_seqlens or None, its version, key, schedule tensor), newest
+# last; the key holds the stream, so a schedule is only ever reused behind the launch that wrote it.
+_sched_cache = []
+_SCHED_CACHE_SIZE = 8
+
+
+def _schedule_workspace(cu: Optional[torch.Tensor], sched_bytes: int, batch: int, tokens: int, device):
+    """(schedule tensor, whether its contents still have to be built).  Eager mode only remembers;
+    while torch.compile traces every call gets a fresh workspace."""
+    if torch.compiler.is_compiling():
+        return torch.empty(sched_bytes, dtype=torch.uint8, device=device), True
+    version = None if cu is None else _version_of(cu)
+    key = (device, torch.cuda.current_stream(device).cuda_stream, batch, tokens, sched_bytes)
+    if cu is None or version is not None:
+        for i in range(len(_sched_cache) - 1, -1, -1):
+            ref, ver, k, sched = _sched_cache[i]
+            if k == key and (ref is None if cu is None else (ref is not None and ref() is cu)):
+                if ver == version:
+                    return sched, False
+                del _sched_cache[i]
+                break
+    sched = torch.empty(sched_bytes, dtype=torch.uint8, device=device)
+    if cu is None or version is not None:
+        _sched_cache[:] = [e for e in _sched_cache if e[0] is None or e[0]() is not None][-(_SCHED_CACHE_SIZE - 1):]
+        _sched_cache.append((None if cu is None else weakref.ref(cu), version, key, sched))
+    return sched, True
 
 
 def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, attend_current: bool,
@@ -359,17 +398,17 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
     o = torch.empty_like(qp)
     rem = torch.empty_like(qp[..., 0])
     table = torch.empty(table_floats if need_table else 0, dtype=torch.float32, device=q.device)
-    sched = torch.empty(sched_bytes, dtype=torch.uint8, device=q.device)
+    sched, build = _schedule_workspace(cu, sched_bytes, B, T, q.device)
     if return_attention:
         weights = torch.zeros(qp.shape[:-1] + (T,), dtype=torch.float32, device=q.device)
         _launch_fwd(fixed, qp, kp, vp, cu, max_len, float(inv_temp), bool(attend_current), product, bool(fused),
-                    o, rem, table, sched, weights=weights)
+                    o, rem, table, sched, weights=weights, build_schedule=build)
     elif fixed:
         _compileable_fwd(qp, kp, vp, float(inv_temp), bool(attend_current), product, bool(fused),
-                         o, rem, table, sched)
+                         o, rem, table, sched, build)
     else:
         _compileable_forward(qp, kp, vp, cu, max_len, float(inv_temp), bool(attend_current), product,
-                             bool(fused), o, rem, table, sched)
+                             bool(fused), o, rem, table, sched, build)
         if VALIDATE and not torch.compiler.is_compiling():
             check_status(sched, table, H, max_len)
     if dpad != d or q.dtype != cdt:
@@ -412,9 +451,11 @@ def _grad_table(like: torch.Tensor) -> torch.Tensor:
 
 
 def release_workspaces() -> None:
-    """Drop the cached gradient tables and host copies of cu_seqlens."""
+    """Drop the cached gradient tables, schedules and host copies of cu_seqlens."""
     _gtab_cache.clear()
     del _host_cu_cache[:]
+    del _sched_cache[:]
+    del _stripped_views[:]
 
 
 def run_backward(q, k, v, do, drem, fixed: bool, state, inv_temp: float, attend_current: bool, dkdv_dtype=None,
