@@ -29,7 +29,7 @@ struct Sizes {
 int check_problem(const sba_problem* p, bool fixed, Sizes* sz) {
   if (p == nullptr) return SBA_E_NULL;
   if (p->dtype != SBA_BF16 && p->dtype != SBA_F16) return SBA_E_DTYPE;
-  if (p->head_dim != 64 && p->head_dim != 128) return SBA_E_HEAD_DIM;
+  if (p->head_dim != 32 && p->head_dim != 64 && p->head_dim != 128) return SBA_E_HEAD_DIM;
   if (p->heads <= 0 || p->tokens < 0 || p->batch <= 0 || p->max_doc_len < 0) return SBA_E_SHAPE;
   if (fixed != ((p->flags & SBA_FIXED_LENGTH) != 0)) return SBA_E_SHAPE;
   if (fixed) {

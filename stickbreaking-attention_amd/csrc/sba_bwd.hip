@@ -605,7 +605,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       lds_barrier();
     };
     auto later = [&](auto slot_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& set) {
-      if constexpr (PROD) bulk(slot_tag, i, xc, dc, xn, dn, set);
+      if constexpr (PROD && D >= 64) bulk(slot_tag, i, xc, dc, xn, dn, set);   // (its eight chunks need 2 * KS >= 8 chain steps)
       else step(std::false_type{}, i, xc, dc, xn, dn, set);
     };
     f32x16 xa, da, xb, db;
@@ -666,12 +666,17 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     }
     // Tile staging by the 256 product threads: asynchronous global -> LDS copies straight into
     // the ring slot, well ahead of the score waves that will read it.
-    using Copy = TileCopy<D, BQ, NPT, false>;
+    // (a 32 x 32 tile is one instruction each for two waves: the other two request nothing, wait
+    // for nothing and meet the copies at the barrier)
+    constexpr int CT = D == 32 ? NPT / 2 : NPT;   // threads that copy tiles
+    const bool copier = ptid < CT;                // (uniform per wave)
+    using Copy = TileCopy<D, BQ, CT, false>;
     constexpr int LOADS_PER_TILE = 2 * Copy::NCH;
     Copy qcopy, gcopy;
     qcopy.init(ptid, qrows.row_bytes);
     gcopy.init(ptid, grows.row_bytes);
     auto fetch = [&](int step) {
+      if (!copier) return;
       qcopy.issue(qrows, q_first + step * BQ, Qs + (step % RING) * QTILE);
       gcopy.issue(grows, q_first + step * BQ, Gs + (step % RING) * QTILE);
     };
@@ -930,6 +935,10 @@ __global__ void __launch_bounds__(NT, 2) bwd_dkdv_tail_kernel(const KArgs a) {
 }
 
 // Explicit instantiations: every (head_dim, attend_current, carry space) variant the launchers use.
+template __global__ void bwd_dq_kernel<32, false, false>(const KArgs);
+template __global__ void bwd_dq_kernel<32, false, true>(const KArgs);
+template __global__ void bwd_dq_kernel<32, true, false>(const KArgs);
+template __global__ void bwd_dq_kernel<32, true, true>(const KArgs);
 template __global__ void bwd_dq_kernel<64, false, false>(const KArgs);
 template __global__ void bwd_dq_kernel<64, false, true>(const KArgs);
 template __global__ void bwd_dq_kernel<64, true, false>(const KArgs);
@@ -942,6 +951,10 @@ template __global__ void bwd_dkdv_tail_kernel<64, false, false>(const KArgs);
 template __global__ void bwd_dkdv_tail_kernel<64, false, true>(const KArgs);
 template __global__ void bwd_dkdv_tail_kernel<64, true, false>(const KArgs);
 template __global__ void bwd_dkdv_tail_kernel<64, true, true>(const KArgs);
+template __global__ void bwd_dkdv_kernel<32, false, false>(const KArgs);
+template __global__ void bwd_dkdv_kernel<32, false, true>(const KArgs);
+template __global__ void bwd_dkdv_kernel<32, true, false>(const KArgs);
+template __global__ void bwd_dkdv_kernel<32, true, true>(const KArgs);
 template __global__ void bwd_dkdv_kernel<64, false, false>(const KArgs);
 template __global__ void bwd_dkdv_kernel<64, false, true>(const KArgs);
 template __global__ void bwd_dkdv_kernel<64, true, false>(const KArgs);
@@ -996,13 +1009,15 @@ static hipError_t launch_dkdv_d(const KArgs& a, bool ac, bool prod, int n_long_m
 
 hipError_t launch_bwd_dq(const KArgs& a, int head_dim, bool ac, bool prod, int n_q_max, hipStream_t s) {
   if (head_dim == 128) return launch_dq_d<128>(a, ac, prod, n_q_max, s);
-  return launch_dq_d<64>(a, ac, prod, n_q_max, s);
+  if (head_dim == 64) return launch_dq_d<64>(a, ac, prod, n_q_max, s);
+  return launch_dq_d<32>(a, ac, prod, n_q_max, s);
 }
 
 hipError_t launch_bwd_dkdv(const KArgs& a, int head_dim, bool ac, bool prod, int n_long_max, int n_last_max,
                            hipStream_t s) {
   if (head_dim == 128) return launch_dkdv_d<128>(a, ac, prod, n_long_max, n_last_max, s);
-  return launch_dkdv_d<64>(a, ac, prod, n_long_max, n_last_max, s);
+  if (head_dim == 64) return launch_dkdv_d<64>(a, ac, prod, n_long_max, n_last_max, s);
+  return launch_dkdv_d<32>(a, ac, prod, n_long_max, n_last_max, s);
 }
 
 }  // inline namespace SBA_ELEM_NS

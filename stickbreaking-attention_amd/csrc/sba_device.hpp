@@ -474,7 +474,8 @@ __device__ __forceinline__ el8 load_frag(const Rows& r, int row, int col_bytes) 
 template <int D>
 __device__ __forceinline__ int swz(int row) {
   if constexpr (D == 128) return ((row & 3) << 2) | ((row >> 2) & 3);
-  else { const int x = (row >> 1) & 7; return ((x & 1) << 2) | (x >> 1); }
+  else if constexpr (D == 64) { const int x = (row >> 1) & 7; return ((x & 1) << 2) | (x >> 1); }
+  else return (row >> 2) & 3;   // 64-byte rows: four rows fill the banks, the next four take the next rotation
 }
 
 template <int D>

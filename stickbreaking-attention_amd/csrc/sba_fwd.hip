@@ -74,15 +74,21 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   for (int ks = 0; ks < KS; ++ks) qf[ks] = load_frag(qrows, qrow, 32 * ks + 16 * h);
 
   // Three-stage ring of K/V tiles: two tiles are in flight while one is consumed.
-  TileCopy<D, BF, NT, true> kcopy, vcopy;
+  // (a 32 x 32 tile is one instruction each for two waves: the other two request nothing, wait for
+  // nothing and meet the copies at the barrier)
+  constexpr int CT = D == 32 ? NT / 2 : NT;   // threads that copy tiles
+  const bool copier = tid < CT;               // (uniform per wave)
+  TileCopy<D, BF, CT, true> kcopy, vcopy;
   kcopy.init(tid, krows.row_bytes);
   vcopy.init(tid, vrows.row_bytes);
-  constexpr int LOADS_PER_TILE = 2 * TileCopy<D, BF, NT, true>::NCH;
-  kcopy.issue(krows, kt_last * BF, Ks);
-  vcopy.issue(vrows, kt_last * BF, Vs);
-  if (kt_last >= 1) {
-    kcopy.issue(krows, (kt_last - 1) * BF, Ks + TILE);
-    vcopy.issue(vrows, (kt_last - 1) * BF, Vs + TILE);
+  constexpr int LOADS_PER_TILE = 2 * TileCopy<D, BF, CT, true>::NCH;
+  if (copier) {
+    kcopy.issue(krows, kt_last * BF, Ks);
+    vcopy.issue(vrows, kt_last * BF, Vs);
+    if (kt_last >= 1) {
+      kcopy.issue(krows, (kt_last - 1) * BF, Ks + TILE);
+      vcopy.issue(vrows, (kt_last - 1) * BF, Vs + TILE);
+    }
   }
 
   f32x16 oacc[DB];
@@ -119,7 +125,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
     // order) can still be in flight; stores in between only make the wait stricter.
     if (kt >= 1) wait_loads<LOADS_PER_TILE>(); else wait_loads<0>();
     lds_barrier();
-    if (kt >= 2) {
+    if (kt >= 2 && copier) {
       kcopy.issue(krows, (kt - 2) * BF, Ks + REFILL * TILE);
       vcopy.issue(vrows, (kt - 2) * BF, Vs + REFILL * TILE);
     }
@@ -203,6 +209,14 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
 }
 
 // Explicit instantiations: every (head_dim, attend_current, carry space) variant the launchers use.
+template __global__ void fwd_kernel<32, false, false, false>(const KArgs);
+template __global__ void fwd_kernel<32, false, false, true>(const KArgs);
+template __global__ void fwd_kernel<32, false, true, false>(const KArgs);
+template __global__ void fwd_kernel<32, false, true, true>(const KArgs);
+template __global__ void fwd_kernel<32, true, false, false>(const KArgs);
+template __global__ void fwd_kernel<32, true, false, true>(const KArgs);
+template __global__ void fwd_kernel<32, true, true, false>(const KArgs);
+template __global__ void fwd_kernel<32, true, true, true>(const KArgs);
 template __global__ void fwd_kernel<64, false, false, false>(const KArgs);
 template __global__ void fwd_kernel<64, false, false, true>(const KArgs);
 template __global__ void fwd_kernel<64, false, true, false>(const KArgs);
@@ -236,10 +250,12 @@ static hipError_t launch_fwd_d(const KArgs& a, bool ac, bool prod, int n_q_max, 
 hipError_t launch_fwd(const KArgs& a, int head_dim, bool ac, bool prod, bool weights, int n_q_max, hipStream_t s) {
   if (weights) {
     if (head_dim == 128) return launch_fwd_d<128, true>(a, ac, prod, n_q_max, s);
-    return launch_fwd_d<64, true>(a, ac, prod, n_q_max, s);
+    if (head_dim == 64) return launch_fwd_d<64, true>(a, ac, prod, n_q_max, s);
+    return launch_fwd_d<32, true>(a, ac, prod, n_q_max, s);
   }
   if (head_dim == 128) return launch_fwd_d<128, false>(a, ac, prod, n_q_max, s);
-  return launch_fwd_d<64, false>(a, ac, prod, n_q_max, s);
+  if (head_dim == 64) return launch_fwd_d<64, false>(a, ac, prod, n_q_max, s);
+  return launch_fwd_d<32, false>(a, ac, prod, n_q_max, s);
 }
 
 }  // inline namespace SBA_ELEM_NS

@@ -41,7 +41,7 @@ VALIDATE = os.environ.get("SBA_VALIDATE", "0") == "1"
 # (tokens, max_seqlens) and errors surface as NaN outputs.
 SYNC_FREE = os.environ.get("SBA_SYNC_FREE", "0") == "1"
 
-SUPPORTED_HEAD_DIMS = (64, 128)
+SUPPORTED_HEAD_DIMS = (32, 64, 128)
 
 # Tile sizes the library's workspace formulas are built on (query tile, dk/dv key tile, table block).
 _BM, _BKV, _BT, _SCHED_HDR, _TILE_WORDS = 128, 128, 32, 16, 8
