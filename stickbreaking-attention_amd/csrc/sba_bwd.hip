@@ -338,7 +338,7 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
 constexpr int NT2 = 512;
 // Head dimensions for which the second group of key tiles (a handful of steps each, most of them on or
 // near the diagonal) goes to bwd_dkdv_tail_kernel instead.
-template <int D> struct TailKernel { static constexpr bool value = D == 64; };
+template <int D> struct TailKernel { static constexpr bool value = D <= 64; };
 constexpr int BQ = 32;     // queries per step of the dk/dv pass
 constexpr int RING = 6;    // Q/dO tile slots: tiles i-1 (products) .. i+4 (in flight) of step i
 constexpr int AHEAD = 4;   // a tile is requested this many steps before the products use it + 1
@@ -799,7 +799,7 @@ __global__ void __launch_bounds__(NT, 2) bwd_dkdv_tail_kernel(const KArgs a) {
     TileCopy<D, QROWS, NT, false> qcopy, gcopy;
     qcopy.init(tid, qrows.row_bytes);
     gcopy.init(tid, grows.row_bytes);
-    qcopy.issue(qrows, q_first, Qs, 32 * nblk);      // (32 rows per instruction: whole query blocks)
+    qcopy.issue(qrows, q_first, Qs, 32 * nblk);      // (32 or 64 rows per instruction of all waves: whole query blocks)
     gcopy.issue(grows, q_first, Gs, 32 * nblk);
   }
   // Wave w of workgroup b takes key block (w + b) mod 4: the block with the most queries behind it
@@ -925,8 +925,8 @@ __global__ void __launch_bounds__(NT, 2) bwd_dkdv_tail_kernel(const KArgs a) {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the reads are done before the next block overwrites the piece
     cur = nxt;
   }
-  // the private piece becomes the output scratch (32 x D elements: exactly its size)
-  static_assert(2 * 32 * 32 == 32 * D, "the staging piece of a wave doubles as its output scratch");
+  // the private piece becomes the output scratch (32 x D elements: at most its size)
+  static_assert(2 * 32 * 32 >= 32 * D, "the staging piece of a wave doubles as its output scratch");
   elem_t* dvb = reinterpret_cast<elem_t*>(a.dv.ptr) + t.batch * a.dv.sb + head * a.dv.sh + tok0 * a.dv.st;
   elem_t* dkb = reinterpret_cast<elem_t*>(a.dk.ptr) + t.batch * a.dk.sb + head * a.dk.sh + tok0 * a.dk.st;
   store_block32<D>(Pt, acc_v, 1.0f, dvb, a.dv.st, k0, L, lane);
@@ -947,6 +947,10 @@ template __global__ void bwd_dq_kernel<128, false, false>(const KArgs);
 template __global__ void bwd_dq_kernel<128, false, true>(const KArgs);
 template __global__ void bwd_dq_kernel<128, true, false>(const KArgs);
 template __global__ void bwd_dq_kernel<128, true, true>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<32, false, false>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<32, false, true>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<32, true, false>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<32, true, true>(const KArgs);
 template __global__ void bwd_dkdv_tail_kernel<64, false, false>(const KArgs);
 template __global__ void bwd_dkdv_tail_kernel<64, false, true>(const KArgs);
 template __global__ void bwd_dkdv_tail_kernel<64, true, false>(const KArgs);
