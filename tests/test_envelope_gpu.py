@@ -81,7 +81,7 @@ def test_fp32_inputs_are_rounded_to_bf16_and_say_so():
         assert_close(name + " (fp32 inputs)", gt, r)
 
 
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [32, 64, 128])
 def test_float16_runs_on_the_float16_kernels(d):
     """float16 q, k, v, grad_o are multiplied as float16 (11 significant bits instead of bfloat16's 8;
     upstream's tl.dot does the same, sb_varlen_fwd.py:42): the operands P and dZ and the outputs are
