@@ -31,6 +31,9 @@ class StickBreakingAttention(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, inv_temp, attend_current=False):
+        # an output nobody differentiates through arrives as None in backward instead of as a tensor of
+        # zeros that PyTorch would have to allocate and fill
+        ctx.set_materialize_grads(False)
         no_grad = not any(ctx.needs_input_grad[:3])
         o, rem, state = _fwd(q, k, v, logit_scale=inv_temp, attend_current=attend_current, no_grad=no_grad)
         table, sched, _cu, max_len, product = state
@@ -45,6 +48,8 @@ class StickBreakingAttention(torch.autograd.Function):
     def backward(ctx, do, drem):
         q, k, v, table, sched = ctx.saved_tensors
         state = (table, sched, None, ctx.max_seqlens, ctx.product)
+        if do is None:          # only rem was used
+            do = torch.zeros_like(q)
         dq, dk, dv = _bwd(do, drem, q, k, v, state, ctx.logit_scale, ctx.attend_current)
         return dq, dk, dv, None, None
 

@@ -77,6 +77,9 @@ class StickBreakingAttention(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, cu_seqlens, max_seqlens, inv_temp, attend_current):
+        # an output nobody differentiates through arrives as None in backward instead of as a tensor of
+        # zeros that PyTorch would have to allocate and fill
+        ctx.set_materialize_grads(False)
         no_grad = not any(ctx.needs_input_grad[:3])
         o, rem, state = varlen_fwd(q, k, v, cu_seqlens, max_seqlens, logit_scale=inv_temp,
                                    attend_current=attend_current, no_grad=no_grad)
@@ -92,6 +95,8 @@ class StickBreakingAttention(torch.autograd.Function):
     def backward(ctx, do, drem):
         q, k, v, table, sched, cu = ctx.saved_tensors
         state = (table, sched, cu, ctx.max_seqlens, ctx.product)
+        if do is None:          # only rem was used
+            do = torch.zeros_like(q)
         dq, dk, dv = varlen_bwd(do, drem, q, k, v, state, ctx.logit_scale, ctx.attend_current)
         return dq, dk, dv, None, None, None, None
 

@@ -448,6 +448,27 @@ def test_malformed_cu_seqlens_are_reported(monkeypatch):
     torch.cuda.synchronize()
 
 
+def test_gradient_through_rem_alone():
+    """Only ``rem`` is differentiated: the gradient of ``o`` arrives as None (the functions do not ask
+    PyTorch to materialise zeros for unused outputs) and must behave as zeros."""
+    from stickbreaking_attention import sb_attn, sb_attn_varlen
+    lengths = [150, 90]
+    q, k, v, _ = orc.make_inputs((2, sum(lengths), 64), 17)
+    drem = torch.randn((2, sum(lengths)), generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+    o, rem = sb_attn_varlen(qg, kg, vg, cu_from_lengths(lengths, device=DEV), max(lengths), zero_start=False)
+    dq, dk, dv = torch.autograd.grad(rem, (qg, kg, vg), drem.to(DEV))
+    torch.cuda.synchronize()
+    ref = oracle_varlen(q, k, v, torch.zeros_like(q), lengths, False, drem=drem)
+    check_all((o.detach(), rem.detach(), dq, dk, dv), ref)
+    qf, kf, vf = (t[None].to(DEV).requires_grad_() for t in (q[:, :150], k[:, :150], v[:, :150]))
+    o2, rem2 = sb_attn(qf, kf, vf)
+    g2 = torch.autograd.grad(rem2, (qf, kf, vf), drem[None, :, :150].to(DEV))
+    torch.cuda.synchronize()
+    for a, b in zip(g2, (dq, dk, dv)):
+        assert torch.equal(a[0], b[:, :150])
+
+
 def test_forward_only_needs_no_table():
     from stickbreaking_attention import sb_attn_varlen
     q, k, v, _ = orc.make_inputs((2, 300, 64), 2)
