@@ -344,8 +344,9 @@ _SCHED_CACHE_SIZE = 8
 
 def _schedule_workspace(cu: Optional[torch.Tensor], sched_bytes: int, batch: int, tokens: int, device):
     """(schedule tensor, whether its contents still have to be built).  Eager mode only remembers;
-    while torch.compile traces every call gets a fresh workspace."""
-    if torch.compiler.is_compiling():
+    while torch.compile traces, and while the stream is being captured into a graph (whose replays
+    must not depend on a tensor this cache may drop), every call gets a workspace of its own."""
+    if torch.compiler.is_compiling() or torch.cuda.is_current_stream_capturing():
         return torch.empty(sched_bytes, dtype=torch.uint8, device=device), True
     version = None if cu is None else _version_of(cu)
     key = (device, torch.cuda.current_stream(device).cuda_stream, batch, tokens, sched_bytes)
@@ -439,7 +440,9 @@ _gtab_cache = {}
 
 
 def _grad_table(like: torch.Tensor) -> torch.Tensor:
-    if torch.compiler.is_compiling():
+    # (a captured graph gets a table of its own, from the graph's memory pool: its replays must not
+    # write into a tensor this cache may have dropped since)
+    if torch.compiler.is_compiling() or torch.cuda.is_current_stream_capturing():
         return torch.empty_like(like)
     key = (like.device, torch.cuda.current_stream(like.device).cuda_stream, like.numel())
     t = _gtab_cache.get(key)

@@ -49,6 +49,11 @@ def test_forward_and_backward_replay_from_a_hip_graph(fused):
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         captured = launch(*static)
+    # the replays must not lean on anything the Python layer remembers between eager calls (schedule,
+    # gradient table): drop all of it and let the allocator hand that memory to someone else
+    _ops.release_workspaces()
+    junk = [torch.full((1 << 18,), -1, dtype=torch.int32, device=DEV) for _ in range(16)]
+    torch.cuda.synchronize()
     for seed in (101, 102, 103):
         fresh = inputs(seed)
         for dst, src in zip(static, fresh):
@@ -59,3 +64,4 @@ def test_forward_and_backward_replay_from_a_hip_graph(fused):
         torch.cuda.synchronize()
         for name, a, b in zip(("o", "rem", "dq", "dk", "dv"), captured, eager):
             assert torch.equal(a, b), f"replay with seed {seed}: {name} differs from the eager launch"
+    del junk
