@@ -74,6 +74,13 @@ extern "C" {
                                    of that sum and adds the terms it implies
                                    (d rem += grad_o . v per row, dv += rem * grad_o).  No
                                    upstream counterpart; must match between fwd and bwd    */
+#define SBA_TABLE_ONLY     32u  /* forward entry points only: write the stick table and nothing
+                                   else (v, o and rem are not looked at and may be null views;
+                                   `stick_table` is required).  For a caller that kept no
+                                   table between forward and backward -- the O(heads x tokens)
+                                   footprint of upstream's neg_log_acc -- and rebuilds it in
+                                   front of sba_*_bwd: same kernel, same bits, about 60 % of
+                                   a forward's time.  No upstream counterpart             */
 
 /* A strided view over [batch, heads, tokens, head_dim]; the last dimension is contiguous.
  * Strides are in ELEMENTS.  For packed variable-length input batch == 1 and stride_b is

@@ -164,8 +164,10 @@ int forward(const sba_problem* p, bool fixed, const void* schedule, size_t sched
   Sizes sz;
   int e = check_problem(p, fixed, &sz);
   if (e) return e;
-  if ((e = check_mat(q, p)) || (e = check_mat(k, p)) || (e = check_mat(v, p)) || (e = check_mat(o, p))) return e;
-  if ((e = check_view(rem, true))) return e;
+  const bool table_only = (p->flags & SBA_TABLE_ONLY) != 0;   // nothing but the carry table is written; v, o, rem are not looked at
+  if (table_only && (stick == nullptr || weights != nullptr)) return SBA_E_NULL;
+  if ((e = check_mat(q, p)) || (e = check_mat(k, p))) return e;
+  if (!table_only && ((e = check_mat(v, p)) || (e = check_mat(o, p)) || (e = check_view(rem, true)))) return e;
   if (weights != nullptr &&
       weights_bytes / sizeof(float) < (size_t)p->batch * p->heads * (size_t)p->tokens * (size_t)p->tokens)
     return SBA_E_WORKSPACE;
@@ -174,7 +176,9 @@ int forward(const sba_problem* p, bool fixed, const void* schedule, size_t sched
   if ((e = fill_common(p, fixed, sz, schedule, sched_bytes, stick != nullptr, table_bytes, &a))) return e;
   if ((e = check_arch())) return e;
   if (sz.rows == 0) return 0;
-  a.q = to_view(q); a.k = to_view(k); a.v = to_view(v); a.o = to_view(o); a.rem = to_view(rem);
+  a.q = to_view(q); a.k = to_view(k);
+  if (table_only) a.v = a.o = a.rem = to_view(k);   // (placeholders: the kernel touches none of them)
+  else { a.v = to_view(v); a.o = to_view(o); a.rem = to_view(rem); }
   a.stick = stick;
   a.weights = weights;
   a.clear_spare = fixed ? 0 : 1;
@@ -184,7 +188,7 @@ int forward(const sba_problem* p, bool fixed, const void* schedule, size_t sched
   {   // (packed input without a single document still launches: the spare workgroups clear the outputs)
     Timer tm(0, s, timed);
     he = (p->dtype == SBA_F16 ? f16::launch_fwd : bf16::launch_fwd)(a, p->head_dim, (p->flags & SBA_ATTEND_CURRENT) != 0,
-                    (p->flags & SBA_PRODUCT_SPACE) != 0, weights != nullptr, sz.n_q_max, s);
+                    (p->flags & SBA_PRODUCT_SPACE) != 0, weights != nullptr ? 1 : (table_only ? 2 : 0), sz.n_q_max, s);
   }
   return (int)he;
 }

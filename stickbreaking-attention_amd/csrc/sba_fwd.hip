@@ -11,12 +11,14 @@
 namespace sba {
 inline namespace SBA_ELEM_NS {
 
-// WOUT: also write the attention weights (fp32, before their bf16 rounding) into a dense
+// MODE 1 (WOUT): also write the attention weights (fp32, before their bf16 rounding) into a dense
 // [tokens x tokens] matrix per (batch, head) -- upstream's `return_attention` debug output
-// (sb_varlen_fwd.py:195-202).  A separate instantiation, so the production kernel carries none
-// of it.
-template <int D, bool AC, bool PROD, bool WOUT>
+// (sb_varlen_fwd.py:195-202).  MODE 2 (TAB): write the carry table and nothing else -- no V tiles,
+// no P.V products, no o, no rem -- for a backward whose forward kept no table.  Separate
+// instantiations, so the production kernel (MODE 0) carries none of it.
+template <int D, bool AC, bool PROD, int MODE>
 __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
+  constexpr bool WOUT = MODE == 1, TAB = MODE == 2;
   constexpr int KS = D / 16;     // contraction steps of K.Q^T
   constexpr int DB = D / 32;     // 32-wide output column blocks of P.V
   constexpr int BF = 32;         // keys per staged tile: one MFMA sub-block
@@ -37,7 +39,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch));   // keep the tile read above the branch
   const bool refused = hdr.x != 0 || (a.stick != nullptr && hdr.w > a.tab_stride);
   if (refused || slot >= hdr.y) {
-    if (a.clear_spare) {
+    if (a.clear_spare && !TAB) {
       int row0, row1;
       unsigned pair;
       spare_rows(refused, slot, hdr.y, sched[SCHED_TOTAL], a.tokens, a.nan_pair, row0, row1, pair);
@@ -81,13 +83,13 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   TileCopy<D, BF, CT, true> kcopy, vcopy;
   kcopy.init(tid, krows.row_bytes);
   vcopy.init(tid, vrows.row_bytes);
-  constexpr int LOADS_PER_TILE = 2 * TileCopy<D, BF, CT, true>::NCH;
+  constexpr int LOADS_PER_TILE = (TAB ? 1 : 2) * TileCopy<D, BF, CT, true>::NCH;
   if (copier) {
     kcopy.issue(krows, kt_last * BF, Ks);
-    vcopy.issue(vrows, kt_last * BF, Vs);
+    if (!TAB) vcopy.issue(vrows, kt_last * BF, Vs);
     if (kt_last >= 1) {
       kcopy.issue(krows, (kt_last - 1) * BF, Ks + TILE);
-      vcopy.issue(vrows, (kt_last - 1) * BF, Vs + TILE);
+      if (!TAB) vcopy.issue(vrows, (kt_last - 1) * BF, Vs + TILE);
     }
   }
 
@@ -127,7 +129,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
     lds_barrier();
     if (kt >= 2 && copier) {
       kcopy.issue(krows, (kt - 2) * BF, Ks + REFILL * TILE);
-      vcopy.issue(vrows, (kt - 2) * BF, Vs + REFILL * TILE);
+      if (!TAB) vcopy.issue(vrows, (kt - 2) * BF, Vs + REFILL * TILE);
     }
     const unsigned short* Kt = Ks + SLOT * TILE;
     const unsigned short* Vt = Vs + SLOT * TILE;
@@ -165,6 +167,7 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
         }
       }
     }
+    if constexpr (TAB) return;
     // P as the A operand of O = P.V: slot s of step tt is key 16*h + 8*tt + s, which the
     // permuted tile keeps in LDS row 16*tt + 8*(s/4) + 4*h + s%4.
     el8 vfr[2][DB];
@@ -194,10 +197,11 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
   // epilogue: rem = what is left of the stick; o rows in the accumulator layout
   const float r = PROD ? carry : fast_exp2(carry);
   if (h == 0 && qvalid) {
-    rb[(int64_t)qrow * a.rem.st] = (elem_t)r;
+    if (!TAB) rb[(int64_t)qrow * a.rem.st] = (elem_t)r;
     // rem in full precision for the backward of the fused output (last plane of the table)
     if (stick != nullptr) stick[(unsigned)(tab_rowplane32(t.doc_len) + qrow)] = r;
   }
+  if constexpr (TAB) return;
   lds_barrier();   // every wave is done with the K/V tiles: their memory becomes the o staging area
   if (a.fuse) {
     // what every caller computes next (upstream tests/test_varlen.py:101): o + rem * v
@@ -209,53 +213,72 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
 }
 
 // Explicit instantiations: every (head_dim, attend_current, carry space) variant the launchers use.
-template __global__ void fwd_kernel<32, false, false, false>(const KArgs);
-template __global__ void fwd_kernel<32, false, false, true>(const KArgs);
-template __global__ void fwd_kernel<32, false, true, false>(const KArgs);
-template __global__ void fwd_kernel<32, false, true, true>(const KArgs);
-template __global__ void fwd_kernel<32, true, false, false>(const KArgs);
-template __global__ void fwd_kernel<32, true, false, true>(const KArgs);
-template __global__ void fwd_kernel<32, true, true, false>(const KArgs);
-template __global__ void fwd_kernel<32, true, true, true>(const KArgs);
-template __global__ void fwd_kernel<64, false, false, false>(const KArgs);
-template __global__ void fwd_kernel<64, false, false, true>(const KArgs);
-template __global__ void fwd_kernel<64, false, true, false>(const KArgs);
-template __global__ void fwd_kernel<64, false, true, true>(const KArgs);
-template __global__ void fwd_kernel<64, true, false, false>(const KArgs);
-template __global__ void fwd_kernel<64, true, false, true>(const KArgs);
-template __global__ void fwd_kernel<64, true, true, false>(const KArgs);
-template __global__ void fwd_kernel<64, true, true, true>(const KArgs);
-template __global__ void fwd_kernel<128, false, false, false>(const KArgs);
-template __global__ void fwd_kernel<128, false, false, true>(const KArgs);
-template __global__ void fwd_kernel<128, false, true, false>(const KArgs);
-template __global__ void fwd_kernel<128, false, true, true>(const KArgs);
-template __global__ void fwd_kernel<128, true, false, false>(const KArgs);
-template __global__ void fwd_kernel<128, true, false, true>(const KArgs);
-template __global__ void fwd_kernel<128, true, true, false>(const KArgs);
-template __global__ void fwd_kernel<128, true, true, true>(const KArgs);
+template __global__ void fwd_kernel<32, false, false, 0>(const KArgs);
+template __global__ void fwd_kernel<32, false, false, 1>(const KArgs);
+template __global__ void fwd_kernel<32, false, true, 0>(const KArgs);
+template __global__ void fwd_kernel<32, false, true, 1>(const KArgs);
+template __global__ void fwd_kernel<32, true, false, 0>(const KArgs);
+template __global__ void fwd_kernel<32, true, false, 1>(const KArgs);
+template __global__ void fwd_kernel<32, true, true, 0>(const KArgs);
+template __global__ void fwd_kernel<32, true, true, 1>(const KArgs);
+template __global__ void fwd_kernel<64, false, false, 0>(const KArgs);
+template __global__ void fwd_kernel<64, false, false, 1>(const KArgs);
+template __global__ void fwd_kernel<64, false, true, 0>(const KArgs);
+template __global__ void fwd_kernel<64, false, true, 1>(const KArgs);
+template __global__ void fwd_kernel<64, true, false, 0>(const KArgs);
+template __global__ void fwd_kernel<64, true, false, 1>(const KArgs);
+template __global__ void fwd_kernel<64, true, true, 0>(const KArgs);
+template __global__ void fwd_kernel<64, true, true, 1>(const KArgs);
+template __global__ void fwd_kernel<128, false, false, 0>(const KArgs);
+template __global__ void fwd_kernel<128, false, false, 1>(const KArgs);
+template __global__ void fwd_kernel<128, false, true, 0>(const KArgs);
+template __global__ void fwd_kernel<128, false, true, 1>(const KArgs);
+template __global__ void fwd_kernel<128, true, false, 0>(const KArgs);
+template __global__ void fwd_kernel<128, true, false, 1>(const KArgs);
+template __global__ void fwd_kernel<128, true, true, 0>(const KArgs);
+template __global__ void fwd_kernel<128, true, true, 1>(const KArgs);
 
-template <int D, bool WOUT>
+template __global__ void fwd_kernel<32, false, false, 2>(const KArgs);
+template __global__ void fwd_kernel<32, false, true, 2>(const KArgs);
+template __global__ void fwd_kernel<32, true, false, 2>(const KArgs);
+template __global__ void fwd_kernel<32, true, true, 2>(const KArgs);
+template __global__ void fwd_kernel<64, false, false, 2>(const KArgs);
+template __global__ void fwd_kernel<64, false, true, 2>(const KArgs);
+template __global__ void fwd_kernel<64, true, false, 2>(const KArgs);
+template __global__ void fwd_kernel<64, true, true, 2>(const KArgs);
+template __global__ void fwd_kernel<128, false, false, 2>(const KArgs);
+template __global__ void fwd_kernel<128, false, true, 2>(const KArgs);
+template __global__ void fwd_kernel<128, true, false, 2>(const KArgs);
+template __global__ void fwd_kernel<128, true, true, 2>(const KArgs);
+
+template <int D, int MODE>
 static hipError_t launch_fwd_d(const KArgs& a, bool ac, bool prod, int n_q_max, hipStream_t s) {
   const dim3 grid((unsigned)n_q_max * (unsigned)a.heads), block(NT);
   if (ac) {
-    if (prod) hipLaunchKernelGGL((fwd_kernel<D, true, true, WOUT>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((fwd_kernel<D, true, false, WOUT>), grid, block, 0, s, a);
+    if (prod) hipLaunchKernelGGL((fwd_kernel<D, true, true, MODE>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((fwd_kernel<D, true, false, MODE>), grid, block, 0, s, a);
   } else {
-    if (prod) hipLaunchKernelGGL((fwd_kernel<D, false, true, WOUT>), grid, block, 0, s, a);
-    else hipLaunchKernelGGL((fwd_kernel<D, false, false, WOUT>), grid, block, 0, s, a);
+    if (prod) hipLaunchKernelGGL((fwd_kernel<D, false, true, MODE>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((fwd_kernel<D, false, false, MODE>), grid, block, 0, s, a);
   }
   return hipGetLastError();
 }
 
-hipError_t launch_fwd(const KArgs& a, int head_dim, bool ac, bool prod, bool weights, int n_q_max, hipStream_t s) {
-  if (weights) {
-    if (head_dim == 128) return launch_fwd_d<128, true>(a, ac, prod, n_q_max, s);
-    if (head_dim == 64) return launch_fwd_d<64, true>(a, ac, prod, n_q_max, s);
-    return launch_fwd_d<32, true>(a, ac, prod, n_q_max, s);
+// mode: 0 = o and rem (and the table when one is given), 1 = the attention weights as well, 2 = the table alone
+hipError_t launch_fwd(const KArgs& a, int head_dim, bool ac, bool prod, int mode, int n_q_max, hipStream_t s) {
+  if (mode == 1) {
+    if (head_dim == 128) return launch_fwd_d<128, 1>(a, ac, prod, n_q_max, s);
+    if (head_dim == 64) return launch_fwd_d<64, 1>(a, ac, prod, n_q_max, s);
+    return launch_fwd_d<32, 1>(a, ac, prod, n_q_max, s);
   }
-  if (head_dim == 128) return launch_fwd_d<128, false>(a, ac, prod, n_q_max, s);
-  if (head_dim == 64) return launch_fwd_d<64, false>(a, ac, prod, n_q_max, s);
-  return launch_fwd_d<32, false>(a, ac, prod, n_q_max, s);
+  if (mode == 2) {
+    if (head_dim == 128) return launch_fwd_d<128, 2>(a, ac, prod, n_q_max, s);
+    if (head_dim == 64) return launch_fwd_d<64, 2>(a, ac, prod, n_q_max, s);
+    return launch_fwd_d<32, 2>(a, ac, prod, n_q_max, s);
+  }
+  if (head_dim == 128) return launch_fwd_d<128, 0>(a, ac, prod, n_q_max, s);
+  if (head_dim == 64) return launch_fwd_d<64, 0>(a, ac, prod, n_q_max, s);
+  return launch_fwd_d<32, 0>(a, ac, prod, n_q_max, s);
 }
 
 }  // inline namespace SBA_ELEM_NS

@@ -52,7 +52,7 @@ hipError_t launch_schedule(const SchedArgs& a, hipStream_t s);
 #endif
 #define SBA_DECLARE_LAUNCHERS(NS)                                                                                \
   SBA_INLINE_##NS namespace NS {                                                                                 \
-  hipError_t launch_fwd(const KArgs& a, int head_dim, bool attend_current, bool product, bool weights,           \
+  hipError_t launch_fwd(const KArgs& a, int head_dim, bool attend_current, bool product, int mode,               \
                         int n_q_max, hipStream_t s);                                                             \
   hipError_t launch_bwd_dq(const KArgs& a, int head_dim, bool attend_current, bool product, int n_q_max,         \
                            hipStream_t s);                                                                       \

@@ -23,6 +23,7 @@ FLAG_CU_INT64 = 2
 FLAG_PRODUCT_SPACE = 4
 FLAG_FIXED_LENGTH = 8
 FLAG_FUSE_REMAINDER = 16
+FLAG_TABLE_ONLY = 32
 
 STATUS_MESSAGES = {
     1: "cu_seqlens is not a non-decreasing sequence within [0, total_tokens]",

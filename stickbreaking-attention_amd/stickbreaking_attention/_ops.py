@@ -41,6 +41,13 @@ VALIDATE = os.environ.get("SBA_VALIDATE", "0") == "1"
 # (tokens, max_seqlens) and errors surface as NaN outputs.
 SYNC_FREE = os.environ.get("SBA_SYNC_FREE", "0") == "1"
 
+# With SBA_RECOMPUTE_TABLE=1 a forward keeps NO carry table for its backward: the backward first runs
+# the table-only variant of the forward kernel (scores and stick, no P.V, no outputs) to rebuild it.
+# What a layer holds between forward and backward is then q, k, v alone -- upstream's
+# O(heads x tokens) footprint -- for about 60 % of a forward pass of extra time per backward; the
+# rebuilt table is one scratch buffer shared by all layers.
+RECOMPUTE_TABLE = os.environ.get("SBA_RECOMPUTE_TABLE", "0") == "1"
+
 SUPPORTED_HEAD_DIMS = (32, 64, 128)
 
 # Tile sizes the library's workspace formulas are built on (query tile, dk/dv key tile, table block).
@@ -214,10 +221,10 @@ def _dtype_code(t: torch.Tensor) -> int:
 
 
 def _problem(q: torch.Tensor, fixed: bool, cu_seqlens: Optional[torch.Tensor], max_doc_len: int,
-             inv_temp: float, attend_current: bool, product: bool, fused: bool):
+             inv_temp: float, attend_current: bool, product: bool, fused: bool, extra_flags: int = 0):
     """The ``sba_problem`` of a launch plus the tensors whose pointers it holds."""
     flags = ((nat.FLAG_ATTEND_CURRENT if attend_current else 0) | (nat.FLAG_PRODUCT_SPACE if product else 0) |
-             (nat.FLAG_FUSE_REMAINDER if fused else 0))
+             (nat.FLAG_FUSE_REMAINDER if fused else 0) | extra_flags)
     if fixed:
         B, H, T, d = q.shape
         return nat.SbaProblem(_dtype_code(q), d, H, B, T, 0, T, flags | nat.FLAG_FIXED_LENGTH,
@@ -243,10 +250,15 @@ def _nbytes(t: Optional[torch.Tensor]) -> int:
 
 def _launch_fwd(fixed: bool, q, k, v, cu_seqlens, max_doc_len: int, logit_scale: float, attend_current: bool,
                 product: bool, fused: bool, o, rem, table, sched, weights=None, build_schedule: bool = True) -> None:
+    """(`o` and `rem` without elements: only the carry table is wanted, SBA_TABLE_ONLY.)"""
     nat.require_gpu(q)
     lib = nat.load()
     q, k, v = _aligned(q), _aligned(k), _aligned(v)
-    prob, _keep = _problem(q, fixed, cu_seqlens, max_doc_len, logit_scale, attend_current, product, fused)
+    table_only = o.numel() == 0 and q.numel() != 0
+    if table_only:
+        o = rem = None
+    prob, _keep = _problem(q, fixed, cu_seqlens, max_doc_len, logit_scale, attend_current, product, fused,
+                           nat.FLAG_TABLE_ONLY if table_only else 0)
     name = ("sba_attn_fwd" if fixed else "sba_varlen_fwd") + ("_weights" if weights is not None else "")
     fn = getattr(lib, name)
     extra = () if weights is None else (weights.data_ptr(), _nbytes(weights))
@@ -398,7 +410,8 @@ def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, 
     # belong to no document are cleared (upstream leaves those uninitialised).
     o = torch.empty_like(qp)
     rem = torch.empty_like(qp[..., 0])
-    table = torch.empty(table_floats if need_table else 0, dtype=torch.float32, device=q.device)
+    keep_table = need_table and not RECOMPUTE_TABLE
+    table = torch.empty(table_floats if keep_table else 0, dtype=torch.float32, device=q.device)
     sched, build = _schedule_workspace(cu, sched_bytes, B, T, q.device)
     if return_attention:
         weights = torch.zeros(qp.shape[:-1] + (T,), dtype=torch.float32, device=q.device)
@@ -434,23 +447,52 @@ def check_status(sched: torch.Tensor, table: Optional[torch.Tensor] = None, head
         raise ValueError("sb_attn_varlen: " + nat.STATUS_MESSAGES.get(status, f"scheduler status {status}"))
 
 
-# One gradient table per (device, stream, size), reused by every backward of that shape: the dk/dv
-# pass of one backward has read it before the dq pass of the next (same stream) writes it.
+# One gradient table (and, with RECOMPUTE_TABLE, one rebuilt stick table) per (device, stream, size),
+# reused by every backward of that shape: the dk/dv pass of one backward has read them before the
+# next backward on the same stream writes them.
 _gtab_cache = {}
 
 
-def _grad_table(like: torch.Tensor) -> torch.Tensor:
+def _scratch_table(numel: int, device, role: str) -> torch.Tensor:
     # (a captured graph gets a table of its own, from the graph's memory pool: its replays must not
     # write into a tensor this cache may have dropped since)
     if torch.compiler.is_compiling() or torch.cuda.is_current_stream_capturing():
-        return torch.empty_like(like)
-    key = (like.device, torch.cuda.current_stream(like.device).cuda_stream, like.numel())
+        return torch.empty(numel, dtype=torch.float32, device=device)
+    key = (device, torch.cuda.current_stream(device).cuda_stream, numel, role)
     t = _gtab_cache.get(key)
     if t is None:
-        if len(_gtab_cache) >= 4:
+        if len(_gtab_cache) >= 8:
             _gtab_cache.clear()
-        t = _gtab_cache[key] = torch.empty_like(like)
+        t = _gtab_cache[key] = torch.empty(numel, dtype=torch.float32, device=device)
     return t
+
+
+def _grad_table(like: torch.Tensor) -> torch.Tensor:
+    return _scratch_table(like.numel(), like.device, "grad")
+
+
+def _rebuild_table(qp, kp, vp, fixed: bool, sched, cu, max_len: int, inv_temp: float, attend_current: bool,
+                   product: bool, fused: bool) -> torch.Tensor:
+    """The carry table of a forward that kept none (RECOMPUTE_TABLE): the forward kernel once more, in
+    the variant that forms the weights' running stick but neither multiplies them with V nor writes
+    o and rem.  Same arithmetic on the same inputs with the same schedule: the same table, bit for bit."""
+    if fixed:
+        B, H, T, _ = qp.shape
+        n_docs, lengths = 0, None
+    else:
+        (H, T, _), B = qp.shape, 1
+        n_docs = cu.numel()
+        cu_vals = host_cu_seqlens(cu)
+        lengths = None if cu_vals is None else _lengths_info(cu_vals, T)[2]
+    _, table_floats = workspace_sizes(fixed, B, H, T, n_docs, max_len, lengths)
+    table = _scratch_table(table_floats, qp.device, "stick")
+    o = torch.empty(0, dtype=qp.dtype, device=qp.device)     # (no elements: only the table is written)
+    rem = torch.empty(0, dtype=qp.dtype, device=qp.device)
+    if fixed:
+        _compileable_fwd(qp, kp, vp, inv_temp, attend_current, product, fused, o, rem, table, sched, False)
+    else:
+        _compileable_forward(qp, kp, vp, cu, max_len, inv_temp, attend_current, product, fused, o, rem, table, sched, False)
+    return table
 
 
 def release_workspaces() -> None:
@@ -477,6 +519,9 @@ def run_backward(q, k, v, do, drem, fixed: bool, state, inv_temp: float, attend_
         if torch.compiler.is_compiling():
             dremp = dremp.contiguous()
     dq, dk, dv = torch.empty_like(qp), torch.empty_like(kp), torch.empty_like(vp)
+    if table.numel() == 0 and RECOMPUTE_TABLE:
+        table = _rebuild_table(qp, kp, vp, fixed, sched, cu, max_len, float(inv_temp), bool(attend_current), product,
+                               bool(fused))
     gtab = _grad_table(table)
     if fixed:
         _compileable_bwd(dop, dremp, qp, kp, vp, float(inv_temp), bool(attend_current), product, bool(fused),

@@ -93,6 +93,32 @@ def test_undersized_workspaces_are_refused_on_the_host():
                             tbl - 4, *[ctypes.byref(vf)] * 3, None) == -6
 
 
+def test_table_only_forward_checks_its_arguments():
+    """SBA_TABLE_ONLY: the stick table is required, v / o / rem may be null views, the weights output
+    cannot be combined with it; the table of the fixed-length op is still size-checked."""
+    lib = nat.load()
+    p = problem(flags=nat.FLAG_PRODUCT_SPACE | nat.FLAG_TABLE_ONLY)
+    need = lib.sba_schedule_bytes(ctypes.byref(p))
+    v = nat.SbaView(0x1000, 0, 128 * 16384, 128)
+    null = nat.SbaView(None, 0, 0, 0)
+    sched = ctypes.c_void_p(0x1000)
+    args = [ctypes.byref(x) for x in (v, v, null, null, null)]
+    assert lib.sba_varlen_fwd(ctypes.byref(p), sched, need, *args, None, 0, None) == -1              # no table
+    assert lib.sba_varlen_fwd(ctypes.byref(p), sched, need, *[ctypes.byref(x) for x in (v, null, null, null, null)],
+                              ctypes.c_void_p(0x1000), 1 << 30, None) == -1                             # k missing
+    # everything the host can check is fine: the call gets as far as looking for a gfx950 device
+    # (-7 here, where there is none) without having asked for v, o or rem
+    # (only where no GPU could take the made-up pointers seriously)
+    if not torch.cuda.is_available():
+        assert lib.sba_varlen_fwd(ctypes.byref(p), sched, need, *args, ctypes.c_void_p(0x1000), 1 << 30, None) == -7
+    pf = problem(batch=4, heads=16, tokens=2048, n_docs=0, max_doc_len=2048, head_dim=64,
+                 flags=nat.FLAG_FIXED_LENGTH | nat.FLAG_TABLE_ONLY, cu_seqlens=None)
+    vf = nat.SbaView(0x1000, 16 * 2048 * 64, 2048 * 64, 64)
+    argsf = [ctypes.byref(x) for x in (vf, vf, null, null, null)]
+    assert lib.sba_attn_fwd(ctypes.byref(pf), sched, lib.sba_schedule_bytes(ctypes.byref(pf)), *argsf,
+                            ctypes.c_void_p(0x1000), lib.sba_table_bytes(ctypes.byref(pf)) - 4, None) == -6
+
+
 @pytest.mark.parametrize("kw,code", [
     (dict(head_dim=50), -2), (dict(dtype=7), -3), (dict(dtype=2, head_dim=50), -2), (dict(heads=0), -4), (dict(batch=2), -4),
     (dict(cu_seqlens=None), -1),

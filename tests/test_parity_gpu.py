@@ -469,6 +469,33 @@ def test_gradient_through_rem_alone():
         assert torch.equal(a[0], b[:, :150])
 
 
+@pytest.mark.parametrize("fixed", [False, True])
+def test_backward_can_rebuild_the_carry_table(fixed, monkeypatch):
+    """SBA_RECOMPUTE_TABLE: the forward keeps no table (a layer holds q, k, v only), the backward runs
+    the forward kernel again to rebuild it.  Same kernels on the same inputs: identical bits."""
+    from stickbreaking_attention import _ops, sb_attn, sb_attn_varlen
+    lengths = [700, 130, 41]
+    shape = (2, 3, 600, 64) if fixed else (3, sum(lengths), 128)
+    q, k, v, do = orc.make_inputs(shape, 55)
+    drem = torch.randn(shape[:-1], generator=torch.Generator().manual_seed(9)).to(torch.bfloat16)
+    cu = cu_from_lengths(lengths, device=DEV)
+
+    def run():
+        qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+        o, rem = sb_attn(qg, kg, vg) if fixed else sb_attn_varlen(qg, kg, vg, cu, max(lengths), zero_start=False)
+        saved = [t for t in o.grad_fn.saved_tensors if t.dtype == torch.float32]
+        grads = torch.autograd.grad((o, rem), (qg, kg, vg), (do.to(DEV), drem.to(DEV)))
+        torch.cuda.synchronize()
+        return (o.detach(), rem.detach()) + grads, sum(t.numel() for t in saved)
+
+    plain, kept = run()
+    monkeypatch.setattr(_ops, "RECOMPUTE_TABLE", True)
+    rebuilt, kept2 = run()
+    assert kept > 0 and kept2 == 0, "with the switch on no fp32 table may be saved for the backward"
+    for name, a, b in zip(("o", "rem", "dq", "dk", "dv"), plain, rebuilt):
+        assert torch.equal(a, b), name
+
+
 def test_forward_only_needs_no_table():
     from stickbreaking_attention import sb_attn_varlen
     q, k, v, _ = orc.make_inputs((2, 300, 64), 2)
