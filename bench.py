@@ -30,8 +30,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X published HBM3E bandwidth
 # WRITE_SIZE x1.0).  Counters cannot be read from inside the process, so these are recorded
 # constants, valid for the library version they were measured with (profiles/c3_hbm_traffic_pmc.txt):
 # any other version of libsba.so reports null.
-MEASURED_TRAFFIC = {"sba_version": 204,
-                    "c3": {"fwd_kernel": 1.089e9, "bwd_dq_kernel": 1.077e9, "bwd_dkdv_kernel": 1.201e9}}
+MEASURED_TRAFFIC = {"sba_version": 205,
+                    "c3": {"fwd_kernel": 1.091e9, "bwd_dq_kernel": 1.077e9, "bwd_dkdv_kernel": 1.201e9}}
 
 KERNELS = ["fwd_kernel", "bwd_dq_kernel", "bwd_dkdv_kernel"]
 
