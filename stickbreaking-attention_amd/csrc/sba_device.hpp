@@ -312,23 +312,20 @@ __device__ __forceinline__ void stick_weights(const f32x16& x, float c, int k0, 
 // instructions on this machine, so 16 exp2 + 4 rcp per lane beat 16 exp2 + 16 rcp.
 // The backward kernels need r = 1/t for every key and keep the plain form (stick_weights).
 //
-// The odds are clamped at 2^30 so that a product of four t stays finite (beta = 1 - 2^-30 there,
-// which in fp32 is 1); a masked key has e = 0: its weight is exactly zero and it leaves the
-// stick exactly as it was, so that nothing of a later token reaches the row.
+// Where a product of four t would leave the fp32 range the odds are clamped at 2^30 (beta =
+// 1 - 2^-30 there, which in fp32 is 1); a masked key has e = 0: its weight is exactly zero and it
+// leaves the stick exactly as it was, so that nothing of a later token reaches the row.
 // ---------------------------------------------------------------------------------------------
-template <bool AC, bool BAND>
-__device__ __forceinline__ void stick_weights_fwd(const f32x16& x, float c, int k0, int qrow, int h,
-                                                  float& carry, float (&p)[16]) {
-  const int lim = qrow - k0 - 16 * h + (AC ? 1 : 0);   // visible keys of a band block: i < lim
+template <bool BAND, bool CLAMP>
+__device__ __forceinline__ float stick_odds(const f32x16& x, float c, int lim, float (&e)[16], float (&inv)[4]) {
   // per group of four keys (register i = key 16*h + i, so a smaller i is an older key):
   // the odds e and inv = 1 / ((1 + e0) (1 + e1) (1 + e2) (1 + e3))
-  float e[16], inv[4];
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int i = 4 * g + j;
-      const float ej = fast_exp2(fminf(c * x[i], 30.0f));
+      const float ej = fast_exp2(CLAMP ? fminf(c * x[i], 30.0f) : c * x[i]);
       e[i] = (BAND && !(i < lim)) ? 0.0f : ej;
     }
     float u = 1.0f + e[4 * g];
@@ -337,7 +334,23 @@ __device__ __forceinline__ void stick_weights_fwd(const f32x16& x, float c, int 
     u = fmaf(u, e[4 * g + 3], u);
     inv[g] = fast_rcp(u);
   }
-  const float total = (inv[0] * inv[1]) * (inv[2] * inv[3]);   // what this lane's 16 keys leave of a stick
+  return (inv[0] * inv[1]) * (inv[2] * inv[3]);   // what this lane's 16 keys leave of a stick
+}
+
+template <bool AC, bool BAND>
+__device__ __forceinline__ void stick_weights_fwd(const f32x16& x, float c, int k0, int qrow, int h,
+                                                  float& carry, float (&p)[16]) {
+  const int lim = qrow - k0 - 16 * h + (AC ? 1 : 0);   // visible keys of a band block: i < lim
+  float e[16], inv[4];
+  // The clamp is only ever needed when a group's product leaves the fp32 range (its reciprocal is
+  // then 0 and the weights a * e would be 0 * inf or plain wrong; an infinite odd next to one that
+  // underflowed to 0 even makes the product NaN): that shows as a lane total that is not a
+  // positive number, so the odds are first formed without it -- sixteen instructions fewer per
+  // block -- and the whole wave repeats them with the clamp in the rare block where some lane's
+  // total is 0 or NaN (a stick that really underflows triggers it too: the repeat then merely
+  // confirms the 0).
+  float total = stick_odds<BAND, false>(x, c, lim, e, inv);
+  if (__builtin_amdgcn_ballot_w64(!(total > 0.0f)) != 0) total = stick_odds<BAND, true>(x, c, lim, e, inv);
   float lo, hi;
   both_halves(total, lo, hi);
   // keys of the h=1 lane (16..31) are newer than those of the h=0 lane
