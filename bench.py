@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X published HBM3E bandwidth
 # constants, valid for the library version they were measured with (profiles/c3_hbm_traffic_pmc.txt):
 # any other version of libsba.so reports null.
 MEASURED_TRAFFIC = {"sba_version": 205,
-                    "c3": {"fwd_kernel": 1.091e9, "bwd_dq_kernel": 1.077e9, "bwd_dkdv_kernel": 1.201e9}}
+                    "c3": {"fwd_kernel": 1.111e9, "bwd_dq_kernel": 1.075e9, "bwd_dkdv_kernel": 1.202e9}}
 
 KERNELS = ["fwd_kernel", "bwd_dq_kernel", "bwd_dkdv_kernel"]
 
