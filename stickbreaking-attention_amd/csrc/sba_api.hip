@@ -150,6 +150,7 @@ int fill_common(const sba_problem* p, bool fixed, const Sizes& sz, const void* s
   }
   a->sched = reinterpret_cast<const int*>(schedule);
   a->kv_list_off = SCHED_HDR + TILE_WORDS * sz.n_q_max;
+  a->n_kv_alloc = sz.n_kv_max;
   a->heads = p->heads;
   a->tokens = p->tokens;
   a->fuse = (p->flags & SBA_FUSE_REMAINDER) ? 1 : 0;

@@ -20,6 +20,7 @@
 // Per-score math (upstream sb_varlen_bwd.py:439-453):
 //   G = A * (do.v - drem),  C = inclusive running sum of G over keys,  dz = G - beta * C,
 //   dq = s * dz K,  dk = s * dz^T Q,  dv = A^T do.
+#include <algorithm>
 #include <type_traits>
 
 #include "sba_kernels.hpp"
@@ -985,7 +986,9 @@ static hipError_t launch_dq_d(const KArgs& a, bool ac, bool prod, int n_q_max, h
 template <int D>
 static hipError_t launch_dkdv_d(const KArgs& a, bool ac, bool prod, int n_long_max, int n_last_max, hipStream_t s) {
   const bool split = TailKernel<D>::value;
-  const unsigned n_main = split ? (unsigned)n_long_max : (unsigned)(n_long_max + n_last_max);
+  // (the two bounds together can exceed the room of the key-tile list, which every workgroup reads
+  // its tile from before it knows the list's true length: never launch past the room)
+  const unsigned n_main = split ? (unsigned)n_long_max : (unsigned)std::min(n_long_max + n_last_max, a.n_kv_alloc);
   if (n_main > 0) {
     const dim3 grid(n_main * (unsigned)a.heads), block(NT2);
     if (ac) {

@@ -12,6 +12,7 @@ struct KArgs {
   View go, grem, dq, dk, dv;   // backward tensors (grem.ptr may be null)
   const int* sched;            // schedule workspace
   int kv_list_off;             // int32 offset of the KV tile list inside `sched`
+  int n_kv_alloc;              // tiles that list has room for (no launch may index it beyond)
   float* stick;                // carry table written by the forward (may be null in fwd): per (row, 32-key block) the
                                // stick left on entering the block; per-row plane: rem in fp32
   float* gtab;                 // gradient prefix table (backward scratch); per-row plane: the full d(rem)

@@ -448,6 +448,16 @@ def test_malformed_cu_seqlens_are_reported(monkeypatch):
     torch.cuda.synchronize()
 
 
+def test_many_documents_at_head_dim_128_stay_inside_the_key_tile_list():
+    """Ten documents in 2112 tokens at head_dim 128: the launch bounds of the dk/dv pass's two tile
+    groups add up to more tiles than the key-tile list has room for, and every workgroup reads its
+    tile before it knows the list's true length -- the grid must stop at the room."""
+    lengths = [292, 2, 403, 193, 151, 369, 257, 244, 161, 0]
+    T = sum(lengths) + 40
+    q, k, v, do = orc.make_inputs((1, T, 128), 1208, dist="upstream")
+    check_all(run_varlen(q, k, v, do, lengths, True, max_seqlens=420), oracle_varlen(q, k, v, do, lengths, True))
+
+
 def test_gradient_through_rem_alone():
     """Only ``rem`` is differentiated: the gradient of ``o`` arrives as None (the functions do not ask
     PyTorch to materialise zeros for unused outputs) and must behave as zeros."""
