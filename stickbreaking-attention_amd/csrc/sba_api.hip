@@ -275,7 +275,7 @@ const char* sba_error_string(int code) {
   switch (code) {
     case 0: return "ok";
     case SBA_E_NULL: return "a required pointer is NULL";
-    case SBA_E_HEAD_DIM: return "head_dim must be 64 or 128";
+    case SBA_E_HEAD_DIM: return "head_dim must be 32, 64 or 128";
     case SBA_E_DTYPE: return "unsupported element type (SBA_BF16 or SBA_F16)";
     case SBA_E_SHAPE: return "negative or inconsistent sizes";
     case SBA_E_STRIDE: return "pointer or stride breaks 16-byte row alignment";

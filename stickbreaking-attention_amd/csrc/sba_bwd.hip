@@ -375,7 +375,10 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63, n = lane & 31, h = lane >> 5;
   const int i16 = lane & 15, blk = (lane >> 4) & 1;
+  // Waves w and w + 4 of a workgroup share a SIMD: every SIMD gets one score wave and one product wave.
+  // (Pairing the score waves on two SIMDs and the product waves on the other two was measured: 1.10 against 0.97 ms.)
   const bool scorer = w < 4;
+  const int rw = w & 3;                              // index of the wave inside its role
 
   const int64_t tok0 = t.tok_start;
   const elem_t* qb = reinterpret_cast<const elem_t*>(a.q.ptr) + t.batch * a.q.sb + head * a.q.sh + tok0 * a.q.st;
@@ -397,7 +400,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   // product wave fills the slots the score wave leaves (measured: 5 % faster than the reverse).
   if (scorer) {
     __builtin_amdgcn_s_setprio(3);
-    const int sb = w;                           // 32-key block of this wave
+    const int sb = rw;                          // 32-key block of this wave
     const int k0 = kt * BKV + 32 * sb;
     const int qr = n;                           // this lane's query row inside a tile
     el8 kf[KS], vf[KS];                      // MFMA row n holds key k0 + kperm(n)
@@ -639,8 +642,8 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     lds_barrier();                        // the product waves' last step
   } else {
     __builtin_amdgcn_s_setprio(0);
-    const int ptid = tid - NPT;
-    const int mat = (w >> 1) & 1, half = w & 1;   // (dv | dk) x 64 keys (two 32-key blocks); all D columns
+    const int ptid = rw * 64 + lane;
+    const int mat = (rw >> 1) & 1, half = rw & 1;   // (dv | dk) x 64 keys (two 32-key blocks); all D columns
     f32x16 acc[2][DB];
 #pragma unroll
     for (int kb2 = 0; kb2 < 2; ++kb2)
@@ -741,7 +744,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     // (the last barrier of the loop has passed: the p/dz staging buffers are free)
     const View& ov = mat ? a.dk : a.dv;
     elem_t* outb = reinterpret_cast<elem_t*>(ov.ptr) + t.batch * ov.sb + head * ov.sh + tok0 * ov.st;
-    unsigned short* scratch = (w & 2 ? Zs : Ps) + (w & 1) * 32 * D;
+    unsigned short* scratch = (rw & 2 ? Zs : Ps) + (rw & 1) * 32 * D;
 #pragma unroll
     for (int kb2 = 0; kb2 < 2; ++kb2)
       store_block32<D>(scratch, acc[kb2], mat ? a.inv_temp : 1.0f, outb, ov.st, kt * BKV + 64 * half + 32 * kb2,

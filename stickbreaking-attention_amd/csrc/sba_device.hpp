@@ -507,6 +507,25 @@ __device__ __forceinline__ int swz_off(int row, int chunk) {   // element offset
 // instruction, STEP = rows all waves cover together).  STEP is a multiple of 16, which the
 // swizzle does not see, and the key permutation turns "+ STEP rows" into a fixed row offset, so
 // ONE per-lane byte offset serves every instruction: the rest of the address is scalar.
+// One wave instruction of such a copy (buffer_load_dwordx4 ... lds): lane l fetches the 16 bytes at
+// byte offset voff + soff of the buffer and the hardware writes them to LDS at dst + 16 * l.
+//
+// Issued through inline assembly on purpose.  The compiler's wait-count pass knows that the
+// builtin form of this instruction writes LDS and, unable to tell one tile slot from another,
+// puts `s_waitcnt vmcnt(0)` in front of the next LDS read it cannot prove disjoint -- that is,
+// in front of the reads of the CURRENT tile, right after the copy of a LATER tile was issued --
+// which makes every tile step wait out a full round trip to memory and turns the prefetch rings
+// of the kernels into plain synchronous loads.  Through inline assembly the copy is invisible to
+// that pass, and the counted waits the kernels place themselves (wait_loads<N>, then a barrier,
+// before any wave reads a slot) are the only ones left.  Those are REQUIRED for correctness:
+// nothing else orders an LDS read after the copy that fills its slot.
+__device__ __forceinline__ void async_copy16(__amdgpu_buffer_rsrc_t rsrc, const unsigned short* dst, int voff, int soff) {
+  const unsigned lds_addr = __builtin_amdgcn_readfirstlane((unsigned)(size_t)dst);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               ::"s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory", "m0");
+}
+
 template <int D, int ROWS, int THREADS, bool KEYS>
 struct TileCopy {
   static constexpr int C8 = D / 8;
@@ -542,18 +561,30 @@ struct TileCopy {
     for (int j = 0; j < NCH; ++j) {
       if (!KEYS && j * STEP >= rows_needed) continue;
       const int soff = __builtin_amdgcn_readfirstlane((row0 + row_delta(j)) * (int)r.row_bytes);
+#ifdef SBA_BUILTIN_DMA
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           r.rsrc, (__attribute__((address_space(3))) void*)(lds_tile + (j * STEP + wave * RPI) * D), 16,
           voff, soff, 0, 0);
+#else
+      async_copy16(r.rsrc, lds_tile + (j * STEP + wave * RPI) * D, voff, soff);
+#endif
     }
   }
 };
 
 // Wait until at most N of this wave's global loads (including asynchronous tile copies) are
 // still in flight.
+// (s_waitcnt immediate of gfx9: vmcnt in bits 3:0 and 15:14, expcnt 6:4 and lgkmcnt 11:8 left at
+// their maxima = not waited for.)  Emitted through the builtin, not inline assembly, so that the
+// compiler's own wait-count bookkeeping sees the wait: after a wait_loads<0>() it knows that none
+// of ITS loads is outstanding and places no further vmcnt waits of its own -- which, with the
+// asynchronous copies invisible to it, would otherwise wait for copies that were meant to stay in
+// flight (a wait for "at most k of my loads" is a wait for "at most k of ALL loads").
 template <int N>
 __device__ __forceinline__ void wait_loads() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+  asm volatile("" ::: "memory");
 }
 
 }  // inline namespace SBA_ELEM_NS

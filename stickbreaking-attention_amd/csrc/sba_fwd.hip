@@ -185,6 +185,10 @@ __global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
     }
   };
 
+  // The Q fragments and both tiles have landed.  (A full wait, so that the compiler's bookkeeping
+  // holds no load of its own when the loop begins: a wait it placed inside the loop for the Q
+  // fragments would, from the second step on, wait for the tile copies issued in between.)
+  wait_loads<0>();
   for (int kt = kt_last;;) {
     tile(std::integral_constant<int, 0>{}, kt);
     if (--kt < 0) break;
