@@ -227,6 +227,27 @@ int sba_attn_bwd(const sba_problem* p, const void* schedule, size_t schedule_siz
 
 /* ---- misc ------------------------------------------------------------------------------- */
 
+/* Launch geometry of a problem: host arithmetic only, nothing is launched and no device is
+ * looked at.  It has no counterpart upstream (Triton computes its grids inside the launchers,
+ * sb_varlen_fwd.py:476-480, sb_varlen_bwd.py:511-513); it exists so that a caller, and this
+ * library's own CPU tests, can check that every tile descriptor a workgroup may read lies inside
+ * the schedule workspace: the compute kernels read the descriptor of their slot before they know
+ * how long the lists really are.
+ *   forward / dq pass: `fwd_tiles` / `dq_tiles` slots of the query-tile list (room: query_list_tiles);
+ *   dk/dv pass: `dkdv_main_tiles` slots of the key-tile list from its start (room: key_list_tiles),
+ *   and `dkdv_tail_tiles` workgroups per head that compare their slot with the list's true length
+ *   before they read it.  `long_tiles_bound` / `tail_tiles_bound` are the bounds on the two groups
+ *   of the key-tile list the grids are derived from.  Offsets and sizes are in int32 words. */
+typedef struct sba_geometry {
+  int query_list_tiles, key_list_tiles;
+  int query_list_word, key_list_word, tile_words;
+  long long schedule_words;
+  int fwd_tiles, dq_tiles;
+  int long_tiles_bound, tail_tiles_bound;
+  int dkdv_main_tiles, dkdv_tail_tiles;
+} sba_geometry;
+int sba_launch_geometry(const sba_problem* p, sba_geometry* out);
+
 int         sba_version(void);
 const char* sba_error_string(int code);
 

@@ -59,6 +59,24 @@ long long table_entries_bound(const sba_problem* p, bool fixed) {
   return (tokens / lmax) * tab_doc_entries((int)lmax) + tab_doc_entries((int)(tokens % lmax));
 }
 
+// Grid bounds of the dk/dv pass.  The second group of the key-tile list holds at most TAIL_TILES
+// tiles of every document.  The first group holds ceil(L / BKV) - 1 tiles of a document of more
+// than TAIL_TILES * BKV tokens and none of a shorter one: at most rows / BKV in all and, with the
+// declared longest document, at most that many per document.  The declaration is checked on the
+// device: a longer document makes every backward kernel return and the outputs NaN.
+int declared_max_doc_len(const sba_problem* p, bool fixed) {
+  return (fixed || p->max_doc_len <= 0 || p->max_doc_len > p->tokens) ? p->tokens : p->max_doc_len;
+}
+struct BwdBounds { int n_long_max, n_tail_max; };
+BwdBounds backward_bounds(const sba_problem* p, bool fixed, const Sizes& sz) {
+  const int max_doc_len = declared_max_doc_len(p, fixed);
+  const long long per_doc = (max_doc_len + BKV - 1) / BKV - kv_tail_tiles(max_doc_len);
+  BwdBounds b;
+  b.n_long_max = (int)std::min<long long>(sz.rows / BKV, per_doc * sz.n_docs);
+  b.n_tail_max = (int)std::min<long long>(sz.n_kv_max, (long long)TAIL_TILES * sz.n_docs);
+  return b;
+}
+
 size_t schedule_bytes(const Sizes& sz) {
   size_t words = SCHED_HDR + TILE_WORDS * ((size_t)sz.n_q_max + sz.n_kv_max) + 6 * (size_t)sz.n_docs + 2;
   return (words * sizeof(int) + 255) & ~(size_t)255;
@@ -215,15 +233,9 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, size_t sche
   a.dq = to_view(dq); a.dk = to_view(dk); a.dv = to_view(dv);
   a.stick = const_cast<float*>(stick);
   a.gtab = gtab;
-  // Grid bounds of the dk/dv pass.  The second group of the key-tile list holds at most TAIL_TILES
-  // tiles of every document.  The first group holds ceil(L / BKV) - 1 tiles of a document of more
-  // than TAIL_TILES * BKV tokens and none of a shorter one: at most rows / BKV in all and, with the
-  // declared longest document, at most that many per document.  The declaration is checked on the
-  // device: a longer document makes every backward kernel return and the outputs NaN.
-  a.max_doc_len = (fixed || p->max_doc_len <= 0 || p->max_doc_len > p->tokens) ? p->tokens : p->max_doc_len;
-  const long long per_doc = (a.max_doc_len + BKV - 1) / BKV - kv_tail_tiles(a.max_doc_len);
-  const int n_long_max = (int)std::min<long long>(sz.rows / BKV, per_doc * sz.n_docs);
-  const int n_tail_max = (int)std::min<long long>(sz.n_kv_max, (long long)TAIL_TILES * sz.n_docs);
+  a.max_doc_len = declared_max_doc_len(p, fixed);
+  const BwdBounds bb = backward_bounds(p, fixed, sz);
+  const int n_long_max = bb.n_long_max, n_tail_max = bb.n_tail_max;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const bool ac = (p->flags & SBA_ATTEND_CURRENT) != 0, prod = (p->flags & SBA_PRODUCT_SPACE) != 0;
   a.clear_spare = fixed ? 0 : 1;
@@ -392,6 +404,29 @@ int sba_varlen_fwd_static(const sba_problem* p, const sba_view* q, const sba_vie
   if ((e = sba_build_schedule(p, sched, SBA_STATIC_SCRATCH_BYTES, stream))) return e;
   return forward(p, false, sched, SBA_STATIC_SCRATCH_BYTES, q, k, v, o, rem, nullptr, 0, nullptr, 0, stream,
                  /*timed=*/false);   // (timing creates events)
+}
+
+int sba_launch_geometry(const sba_problem* p, sba_geometry* out) {
+  Sizes sz;
+  const bool fixed = p != nullptr && (p->flags & SBA_FIXED_LENGTH) != 0;
+  int e = check_problem(p, fixed, &sz);
+  if (e) return e;
+  if (out == nullptr) return SBA_E_NULL;
+  const BwdBounds bb = backward_bounds(p, fixed, sz);
+  const DkdvGrid g = dkdv_grid(has_dkdv_tail_kernel(p->head_dim), bb.n_long_max, bb.n_tail_max, sz.n_kv_max);
+  out->query_list_tiles = sz.n_q_max;
+  out->key_list_tiles = sz.n_kv_max;
+  out->query_list_word = SCHED_HDR;
+  out->key_list_word = SCHED_HDR + TILE_WORDS * sz.n_q_max;
+  out->tile_words = TILE_WORDS;
+  out->schedule_words = (long long)(schedule_bytes(sz) / sizeof(int));
+  out->fwd_tiles = sz.n_q_max;     // forward and dq pass: one workgroup per slot of the query-tile list and head
+  out->dq_tiles = sz.n_q_max;
+  out->long_tiles_bound = bb.n_long_max;
+  out->tail_tiles_bound = bb.n_tail_max;
+  out->dkdv_main_tiles = g.main_tiles;
+  out->dkdv_tail_tiles = g.tail_tiles;
+  return 0;
 }
 
 void sba_set_timing(int on) { g_timing.store(on); }

@@ -422,24 +422,31 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     // diagonal of P (which is otherwise zero, or p_jj with attend_current), at no extra traffic.
     float rem_own = 0.0f;
     if (a.fuse && k0 + n < t.doc_len) rem_own = a.stick[tab_rowval + k0 + n];
-    // Per-row carries of a step, branch-free: the address is clamped into the document and the
-    // value replaced by the neutral element past its end (those rows have zero Q and dO).
-    // `request` only issues the loads; `settle` applies the end-of-document selection.  They are
-    // kept apart so that nothing consumes (and therefore waits for) a loaded value until a
-    // whole step after the request.
+    // Per-row carries of a step.  The three runs of rows this wave reads (its block's rows of the two
+    // tables and the per-row plane of the gradient table) are buffer resources, so that a lane
+    // addresses them with a 32-bit byte offset: two vector instructions per step instead of 64-bit
+    // address arithmetic per load.  The row is clamped into the document; rows past its end then
+    // carry the values of its last row, which is harmless: their Q and dO rows are zero (the tile
+    // copies fill them with zeros), so whatever finite p and dz they produce adds nothing to dk, dv.
+    const unsigned run_bytes = (unsigned)t.doc_len * 4u;   // (rows of one block: at most doc_len)
+    const __amdgpu_buffer_rsrc_t stick_rs = __builtin_amdgcn_make_buffer_rsrc(a.stick + tab, 0, run_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t gtab_rs = __builtin_amdgcn_make_buffer_rsrc(a.gtab + tab, 0, run_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t drem_rs = __builtin_amdgcn_make_buffer_rsrc(a.gtab + tab_rowval, 0, run_bytes, 0x00020000);
+    const int row4 = 4 * (q_first + qr), last4 = 4 * (t.doc_len - 1);
+    // `request` only issues the loads; nothing consumes (and therefore waits for) a loaded value
+    // until `settle`, a whole step or more after the request.
     struct Raw { float e, g, d; };
     auto request = [&](int step, Raw& r) {
-      const int qrow = q_first + step * BQ + qr;
-      const int qc = qrow < t.doc_len ? qrow : t.doc_len - 1;
-      r.e = a.stick[tab + qc];
-      r.g = a.gtab[tab + qc];
-      r.d = a.gtab[tab_rowval + qc];
+      const int off = min(row4 + step * (4 * BQ), last4);
+      r.e = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(stick_rs, off, 0, 0));
+      r.g = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(gtab_rs, off, 0, 0));
+      r.d = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(drem_rs, off, 0, 0));
     };
     auto settle = [&](int step, const Raw& r, float& ce, float& cc, float& d_r) {
-      const bool ok = q_first + step * BQ + qr < t.doc_len;
-      ce = ok ? r.e : (PROD ? 1.0f : 0.0f);
-      cc = ok ? r.g : 0.0f;
-      d_r = ok ? r.d : 0.0f;
+      (void)step;
+      ce = r.e;
+      cc = r.g;
+      d_r = r.d;
     };
     // The row-read offsets of this lane inside a tile (chunk 2*ks + h of row qr).
     int roff[KS];
@@ -988,10 +995,9 @@ static hipError_t launch_dq_d(const KArgs& a, bool ac, bool prod, int n_q_max, h
 // n_long_max / n_last_max: upper bounds on the key tiles of the first / second group of the list.
 template <int D>
 static hipError_t launch_dkdv_d(const KArgs& a, bool ac, bool prod, int n_long_max, int n_last_max, hipStream_t s) {
-  const bool split = TailKernel<D>::value;
-  // (the two bounds together can exceed the room of the key-tile list, which every workgroup reads
-  // its tile from before it knows the list's true length: never launch past the room)
-  const unsigned n_main = split ? (unsigned)n_long_max : (unsigned)std::min(n_long_max + n_last_max, a.n_kv_alloc);
+  static_assert(TailKernel<D>::value == (D <= 64), "has_dkdv_tail_kernel() states the same rule for the host");
+  const DkdvGrid g = dkdv_grid(TailKernel<D>::value, n_long_max, n_last_max, a.n_kv_alloc);
+  const unsigned n_main = (unsigned)g.main_tiles;
   if (n_main > 0) {
     const dim3 grid(n_main * (unsigned)a.heads), block(NT2);
     if (ac) {
@@ -1003,8 +1009,8 @@ static hipError_t launch_dkdv_d(const KArgs& a, bool ac, bool prod, int n_long_m
     }
   }
   if constexpr (TailKernel<D>::value) {
-    if (n_last_max > 0) {
-      const dim3 grid((unsigned)n_last_max * (unsigned)a.heads), block(NT);
+    if (g.tail_tiles > 0) {
+      const dim3 grid((unsigned)g.tail_tiles * (unsigned)a.heads), block(NT);
       if (ac) {
         if (prod) hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, true, true>), grid, block, 0, s, a);
         else hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, true, false>), grid, block, 0, s, a);

@@ -42,6 +42,21 @@ struct SchedArgs {
 
 hipError_t launch_schedule(const SchedArgs& a, hipStream_t s);
 
+// Key-tile slots the two kernels of the dk/dv pass are launched over (one workgroup per slot and
+// head).  Every workgroup of the main kernel reads the tile descriptor of its slot BEFORE it knows
+// how many tiles the list really holds, so the main grid must never exceed the room of the list
+// (n_kv_alloc); the tail kernel compares its slot with the true length first.  Head dimensions
+// without a tail kernel give both groups of the list to the main kernel.
+struct DkdvGrid { int main_tiles, tail_tiles; };
+inline DkdvGrid dkdv_grid(bool has_tail_kernel, int n_long_max, int n_last_max, int n_kv_alloc) {
+  DkdvGrid g;
+  g.main_tiles = has_tail_kernel ? (n_long_max < n_kv_alloc ? n_long_max : n_kv_alloc)
+                                 : (n_long_max + n_last_max < n_kv_alloc ? n_long_max + n_last_max : n_kv_alloc);
+  g.tail_tiles = has_tail_kernel ? n_last_max : 0;
+  return g;
+}
+inline bool has_dkdv_tail_kernel(int head_dim) { return head_dim <= 64; }
+
 // One set of compute launchers per element type (sba_fwd.hip and sba_bwd.hip are compiled once
 // for each, see SBA_ELEM_NS).
 #ifdef SBA_ELEM_F16

@@ -44,11 +44,21 @@ class SbaProblem(ctypes.Structure):
                 ("inv_temp", ctypes.c_float), ("cu_seqlens", ctypes.c_void_p)]
 
 
+class SbaGeometry(ctypes.Structure):
+    _fields_ = [("query_list_tiles", ctypes.c_int), ("key_list_tiles", ctypes.c_int),
+                ("query_list_word", ctypes.c_int), ("key_list_word", ctypes.c_int), ("tile_words", ctypes.c_int),
+                ("schedule_words", ctypes.c_longlong),
+                ("fwd_tiles", ctypes.c_int), ("dq_tiles", ctypes.c_int),
+                ("long_tiles_bound", ctypes.c_int), ("tail_tiles_bound", ctypes.c_int),
+                ("dkdv_main_tiles", ctypes.c_int), ("dkdv_tail_tiles", ctypes.c_int)]
+
+
 EXPORTS = (
     "sba_version", "sba_error_string", "sba_schedule_bytes", "sba_table_bytes", "sba_table_bytes_for_lengths",
     "sba_build_schedule",
     "sba_varlen_fwd", "sba_varlen_bwd", "sba_attn_fwd", "sba_attn_bwd", "sba_set_timing",
     "sba_last_kernel_ms", "sba_varlen_fwd_weights", "sba_attn_fwd_weights", "sba_varlen_fwd_static",
+    "sba_launch_geometry",
 )
 
 _lib = None
@@ -72,6 +82,8 @@ def load():
         lib.sba_version.restype = ctypes.c_int
         lib.sba_error_string.restype = ctypes.c_char_p
         lib.sba_error_string.argtypes = [ctypes.c_int]
+        lib.sba_launch_geometry.restype = ctypes.c_int
+        lib.sba_launch_geometry.argtypes = [ctypes.POINTER(SbaProblem), ctypes.POINTER(SbaGeometry)]
         lib.sba_schedule_bytes.restype = ctypes.c_size_t
         lib.sba_schedule_bytes.argtypes = [P]
         lib.sba_table_bytes.restype = ctypes.c_size_t

@@ -246,3 +246,98 @@ def test_python_table_formula_with_lengths_matches_the_library():
     arr = (ctypes.c_int64 * len(lengths))(*lengths)
     _, table = _ops.workspace_sizes(False, 1, p.heads, p.tokens, len(lengths), 0, lengths)
     assert 4 * table == lib.sba_table_bytes_for_lengths(ctypes.byref(p), arr, len(lengths))
+
+
+# ---------------------------------------------------------------------------------------------
+# Launch geometry: every tile descriptor a workgroup can read lies inside the schedule workspace.
+# The forward, dq and dk/dv kernels fetch the descriptor of their slot BEFORE they compare the slot
+# with the true length of the list (one round trip to memory instead of two), so the grids must
+# stay inside the room of the lists whatever the documents are.  The library exports the grids it
+# would launch (sba_launch_geometry, the same functions the launchers call).
+# ---------------------------------------------------------------------------------------------
+def _geometry(**kw):
+    lib = nat.load()
+    p = problem(**kw)
+    g = nat.SbaGeometry()
+    rc = lib.sba_launch_geometry(ctypes.byref(p), ctypes.byref(g))
+    assert rc == 0, rc
+    assert g.schedule_words * 4 == lib.sba_schedule_bytes(ctypes.byref(p))
+    return g
+
+
+def _check_geometry(g, n_docs):
+    # the two lists and the per-document arrays behind them fit the workspace
+    assert g.query_list_word == 16 and g.tile_words == 8
+    assert g.key_list_word == g.query_list_word + g.tile_words * g.query_list_tiles
+    lists_end = g.key_list_word + g.tile_words * g.key_list_tiles
+    assert lists_end + 6 * n_docs + 2 <= g.schedule_words
+    # query-tile-owned kernels: slots 0 .. fwd_tiles-1 of the query list
+    assert 0 <= g.fwd_tiles <= g.query_list_tiles and 0 <= g.dq_tiles <= g.query_list_tiles
+    # dk/dv main kernel: slots 0 .. dkdv_main_tiles-1 of the key list, read unconditionally
+    assert 0 <= g.dkdv_main_tiles <= g.key_list_tiles
+    assert g.key_list_word + g.tile_words * g.dkdv_main_tiles <= g.schedule_words
+    # (the tail kernel checks its slot against the true list length before reading: any grid is safe)
+    assert g.dkdv_tail_tiles >= 0
+
+
+def _tiles(lengths, rows):
+    return sum(-(-n // rows) for n in lengths)
+
+
+def _tail_tiles(n):
+    nkv = -(-n // 128)
+    return nkv if n <= 2 * 128 else 1
+
+
+def test_every_launch_stays_inside_the_schedule_workspace():
+    import random
+    rng = random.Random(20261125)
+    cases = [(0, 0, 0), (128, 0, 0), (128, 1, 128), (1, 1, 1), (2112, 10, 2112), (16384, 8, 4096), (16384, 207, 256),
+             (65536, 6, 32768), (5, 9, 1), (100, 300, 0), (4096, 1, 1), (4096, 1, 99999)]
+    for _ in range(3000):
+        tokens = rng.choice([rng.randint(0, 300), rng.randint(0, 5000), rng.randint(0, 70000)])
+        n_docs = rng.choice([0, 1, rng.randint(0, 12), rng.randint(0, 400)])
+        mdl = rng.choice([0, 1, rng.randint(0, max(tokens, 1)), tokens, tokens + 7])
+        cases.append((tokens, n_docs, mdl))
+    for tokens, n_docs, mdl in cases:
+        for d in (32, 64, 128):
+            g = _geometry(tokens=tokens, n_docs=n_docs, max_doc_len=mdl, head_dim=d, heads=3)
+            _check_geometry(g, n_docs)
+            # what an earlier version launched at head_dim 128 (both bounds added, no clamp) does NOT stay inside:
+            # the test must be able to tell the difference
+    g = _geometry(tokens=2112, n_docs=10, max_doc_len=2112, head_dim=128, heads=3)
+    assert g.long_tiles_bound + g.tail_tiles_bound > g.key_list_tiles >= g.dkdv_main_tiles
+    # fixed length: batch documents of `tokens` tokens each
+    for batch, tokens in [(1, 1), (4, 2048), (3, 500), (2, 16384), (7, 129)]:
+        for d in (32, 64, 128):
+            g = _geometry(batch=batch, tokens=tokens, n_docs=0, max_doc_len=tokens, head_dim=d, heads=2,
+                          flags=nat.FLAG_FIXED_LENGTH, cu_seqlens=None)
+            _check_geometry(g, batch)
+            assert g.fwd_tiles >= batch * -(-tokens // 128)
+
+
+def test_launch_bounds_cover_every_split_into_documents():
+    """The grids are upper bounds: whatever documents fill the token axis, their query tiles, key tiles
+    and the two groups of the key-tile list fit what would be launched (no tile is ever dropped)."""
+    import random
+    rng = random.Random(7)
+    for _ in range(1500):
+        n_docs = rng.choice([1, 2, rng.randint(1, 10), rng.randint(1, 250)])
+        mode = rng.random()
+        if mode < 0.3: lengths = [rng.randint(0, 300) for _ in range(n_docs)]
+        elif mode < 0.6: lengths = [rng.choice([0, 1, 127, 128, 129, 255, 256, 257, 384, 385, 1000]) for _ in range(n_docs)]
+        else: lengths = [int(2 ** rng.uniform(0, 13)) for _ in range(n_docs)]
+        tokens = sum(lengths) + rng.choice([0, 0, 5, 300])      # rows behind the last document are allowed
+        mdl = max(lengths)
+        for d in (64, 128):
+            g = _geometry(tokens=tokens, n_docs=n_docs, max_doc_len=mdl, head_dim=d, heads=1)
+            assert _tiles(lengths, 128) <= g.fwd_tiles
+            n_kv = _tiles(lengths, 128)
+            assert n_kv <= g.key_list_tiles
+            n_tail = sum(_tail_tiles(n) for n in lengths if n > 0)
+            n_long = n_kv - n_tail
+            assert n_long <= g.long_tiles_bound and n_tail <= g.tail_tiles_bound
+            if d == 128:
+                assert n_kv <= g.dkdv_main_tiles           # one kernel takes both groups
+            else:
+                assert n_long <= g.dkdv_main_tiles and n_tail <= g.dkdv_tail_tiles
