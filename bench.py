@@ -185,12 +185,17 @@ def measure(name, steps, warmup, args, torch, lib, lengths_override=None):
     torch.cuda.synchronize()
     ms_fwd = (time.perf_counter() - t0) * 1e3 / steps
 
-    # per-kernel durations: HIP events recorded by the library on the stream it launches on
+    # per-kernel durations: HIP events recorded by the library on the stream it launches on.  The
+    # library keeps the events of the most recent launch of each kernel, and reading them waits for
+    # that launch, so each sample is the LAST of three steps queued back to back: the kernels that are
+    # measured run behind a busy queue exactly as the steps of the timed loop above do, not behind a
+    # host wait.
     lib.sba_set_timing(1)
     acc = [0.0, 0.0, 0.0]
     reps = 10
     for _ in range(reps):
-        step()
+        for _ in range(3):
+            step()
         for i in range(3):
             acc[i] += lib.sba_last_kernel_ms(i)   # waits for that kernel of the step just queued
     lib.sba_set_timing(0)

@@ -18,6 +18,7 @@ import functools
 import math
 import os
 import warnings
+import threading
 import weakref
 from typing import Optional, Sequence, Tuple
 
@@ -100,6 +101,11 @@ def workspace_sizes(fixed: bool, batch: int, heads: int, tokens: int, n_docs: in
     return (4 * words + 255) & ~255, heads * entries
 
 
+# One lock for the module-level caches below (host copies of cu_seqlens, views without the leading
+# zero, schedules, scratch tables): PyTorch runs the backward on its own autograd thread, so the
+# forward thread and the backward thread reach them concurrently.
+_cache_lock = threading.RLock()
+
 # cu_seqlens tensors already copied to the host: (weak reference, version, tuple of values), newest last
 _host_cu_cache = []
 _HOST_CU_CACHE_SIZE = 8
@@ -128,20 +134,27 @@ def host_cu_seqlens(cu_seqlens: torch.Tensor, allow_sync: bool = True) -> Option
     if torch.compiler.is_compiling():
         return None
     version = _version_of(cu_seqlens)
-    if version is not None:
-        for i in range(len(_host_cu_cache) - 1, -1, -1):
-            ref, ver, vals = _host_cu_cache[i]
-            if ref() is cu_seqlens:
-                if ver == version:
-                    return vals
-                del _host_cu_cache[i]
-                break
+    with _cache_lock:
+        if version is not None:
+            for i in range(len(_host_cu_cache) - 1, -1, -1):
+                ref, ver, vals = _host_cu_cache[i]
+                if ref() is cu_seqlens:
+                    if ver == version:
+                        return vals
+                    del _host_cu_cache[i]
+                    break
     if cu_seqlens.is_cuda and (not allow_sync or SYNC_FREE):
+        return None
+    # A device-to-host copy synchronises, which a stream that is being captured into a graph does
+    # not survive: values not already known stay unknown there (worst-case table size, checks on
+    # the device), exactly as with SBA_SYNC_FREE.
+    if cu_seqlens.is_cuda and torch.cuda.is_current_stream_capturing():
         return None
     vals = tuple(int(x) for x in cu_seqlens.tolist())   # the one synchronisation per tensor
     if version is not None:
-        _host_cu_cache[:] = [e for e in _host_cu_cache if e[0]() is not None][-(_HOST_CU_CACHE_SIZE - 1):]
-        _host_cu_cache.append((weakref.ref(cu_seqlens), version, vals))
+        with _cache_lock:
+            _host_cu_cache[:] = [e for e in _host_cu_cache if e[0]() is not None][-(_HOST_CU_CACHE_SIZE - 1):]
+            _host_cu_cache.append((weakref.ref(cu_seqlens), version, vals))
     return vals
 
 
@@ -151,8 +164,9 @@ def remember_host_cu(cu_seqlens: torch.Tensor, vals: Sequence[int]) -> None:
     version = _version_of(cu_seqlens)
     if version is None or torch.compiler.is_compiling():
         return
-    _host_cu_cache[:] = [e for e in _host_cu_cache if e[0]() is not None][-(_HOST_CU_CACHE_SIZE - 1):]
-    _host_cu_cache.append((weakref.ref(cu_seqlens), version, vals if isinstance(vals, tuple) else tuple(int(x) for x in vals)))
+    with _cache_lock:
+        _host_cu_cache[:] = [e for e in _host_cu_cache if e[0]() is not None][-(_HOST_CU_CACHE_SIZE - 1):]
+        _host_cu_cache.append((weakref.ref(cu_seqlens), version, vals if isinstance(vals, tuple) else tuple(int(x) for x in vals)))
 
 
 def _doc_lengths(cu_vals: Sequence[int], tokens: int) -> Tuple[int, ...]:
@@ -362,19 +376,20 @@ def _schedule_workspace(cu: Optional[torch.Tensor], sched_bytes: int, batch: int
         return torch.empty(sched_bytes, dtype=torch.uint8, device=device), True
     version = None if cu is None else _version_of(cu)
     key = (device, torch.cuda.current_stream(device).cuda_stream, batch, tokens, sched_bytes)
-    if cu is None or version is not None:
-        for i in range(len(_sched_cache) - 1, -1, -1):
-            ref, ver, k, sched = _sched_cache[i]
-            if k == key and (ref is None if cu is None else (ref is not None and ref() is cu)):
-                if ver == version:
-                    return sched, False
-                del _sched_cache[i]
-                break
-    sched = torch.empty(sched_bytes, dtype=torch.uint8, device=device)
-    if cu is None or version is not None:
-        _sched_cache[:] = [e for e in _sched_cache if e[0] is None or e[0]() is not None][-(_SCHED_CACHE_SIZE - 1):]
-        _sched_cache.append((None if cu is None else weakref.ref(cu), version, key, sched))
-    return sched, True
+    with _cache_lock:
+        if cu is None or version is not None:
+            for i in range(len(_sched_cache) - 1, -1, -1):
+                ref, ver, k, sched = _sched_cache[i]
+                if k == key and (ref is None if cu is None else (ref is not None and ref() is cu)):
+                    if ver == version:
+                        return sched, False
+                    del _sched_cache[i]
+                    break
+        sched = torch.empty(sched_bytes, dtype=torch.uint8, device=device)
+        if cu is None or version is not None:
+            _sched_cache[:] = [e for e in _sched_cache if e[0] is None or e[0]() is not None][-(_SCHED_CACHE_SIZE - 1):]
+            _sched_cache.append((None if cu is None else weakref.ref(cu), version, key, sched))
+        return sched, True
 
 
 def run_forward(q, k, v, fixed: bool, cu_seqlens, max_seqlens, inv_temp: float, attend_current: bool,
@@ -447,10 +462,21 @@ def check_status(sched: torch.Tensor, table: Optional[torch.Tensor] = None, head
         raise ValueError("sb_attn_varlen: " + nat.STATUS_MESSAGES.get(status, f"scheduler status {status}"))
 
 
-# One gradient table (and, with RECOMPUTE_TABLE, one rebuilt stick table) per (device, stream, size),
-# reused by every backward of that shape: the dk/dv pass of one backward has read them before the
-# next backward on the same stream writes them.
+# One gradient table (and, with RECOMPUTE_TABLE, one rebuilt stick table) per (device, stream), shared by
+# every backward on that stream: the dk/dv pass of one backward has read them before the next backward
+# on the same stream writes them.  The buffer only ever grows: packed-document training changes
+# cu_seqlens, and with it the exact table size, with every batch, and a buffer per size would
+# allocate on every step and pin what it allocated before.  A request gets the first `numel` floats
+# of the buffer; growth goes to the next eighth of a power of two, and by at least a quarter, so that a
+# sequence of slowly growing sizes does not reallocate every time.
 _gtab_cache = {}
+
+
+def _size_class(numel: int) -> int:
+    if numel <= 1 << 16:
+        return 1 << 16
+    step = 1 << max(0, numel.bit_length() - 4)     # an eighth of the power of two below numel
+    return (numel + step - 1) // step * step
 
 
 def _scratch_table(numel: int, device, role: str) -> torch.Tensor:
@@ -458,13 +484,15 @@ def _scratch_table(numel: int, device, role: str) -> torch.Tensor:
     # write into a tensor this cache may have dropped since)
     if torch.compiler.is_compiling() or torch.cuda.is_current_stream_capturing():
         return torch.empty(numel, dtype=torch.float32, device=device)
-    key = (device, torch.cuda.current_stream(device).cuda_stream, numel, role)
-    t = _gtab_cache.get(key)
-    if t is None:
-        if len(_gtab_cache) >= 8:
-            _gtab_cache.clear()
-        t = _gtab_cache[key] = torch.empty(numel, dtype=torch.float32, device=device)
-    return t
+    key = (device, torch.cuda.current_stream(device).cuda_stream, role)
+    with _cache_lock:
+        buf = _gtab_cache.get(key)
+        if buf is None or buf.numel() < numel:
+            grown = 0 if buf is None else buf.numel() * 5 // 4     # outgrown once: leave room for the next batch too
+            _gtab_cache.pop(key, None)      # (the old buffer goes back to the allocator before the new one is asked for)
+            buf = None
+            buf = _gtab_cache[key] = torch.empty(_size_class(max(numel, grown)), dtype=torch.float32, device=device)
+        return buf[:numel]
 
 
 def _grad_table(like: torch.Tensor) -> torch.Tensor:
@@ -497,10 +525,11 @@ def _rebuild_table(qp, kp, vp, fixed: bool, sched, cu, max_len: int, inv_temp: f
 
 def release_workspaces() -> None:
     """Drop the cached gradient tables, schedules and host copies of cu_seqlens."""
-    _gtab_cache.clear()
-    del _host_cu_cache[:]
-    del _sched_cache[:]
-    del _stripped_views[:]
+    with _cache_lock:
+        _gtab_cache.clear()
+        del _host_cu_cache[:]
+        del _sched_cache[:]
+        del _stripped_views[:]
 
 
 def run_backward(q, k, v, do, drem, fixed: bool, state, inv_temp: float, attend_current: bool, dkdv_dtype=None,

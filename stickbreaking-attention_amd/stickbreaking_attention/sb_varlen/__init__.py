@@ -42,8 +42,12 @@ def _starts_at_zero(cu_seqlens) -> bool:
     if torch.compiler.is_compiling():
         return bool(cu_seqlens[0] == 0)
     vals = _ops.host_cu_seqlens(cu_seqlens)
-    if vals is None:                      # SBA_SYNC_FREE: upstream's assertion still needs this one value
-        return bool(cu_seqlens[0] == 0)
+    if vals is None:
+        # While the stream is being captured into a graph no value can be read back (a
+        # synchronisation would end the capture): the caller's zero_start=True is taken at its word.
+        if cu_seqlens.is_cuda and torch.cuda.is_current_stream_capturing():
+            return True
+        return bool(cu_seqlens[0] == 0)   # SBA_SYNC_FREE: upstream's assertion still needs this one value
     return len(vals) > 0 and vals[0] == 0
 
 
@@ -55,22 +59,23 @@ def _strip_leading_zero(cu_seqlens):
     if torch.compiler.is_compiling():
         return cu_seqlens[1:]
     version = _ops._version_of(cu_seqlens)
-    if version is not None:
-        for i in range(len(_ops._stripped_views) - 1, -1, -1):
-            ref, ver, view = _ops._stripped_views[i]
-            if ref() is cu_seqlens:
-                if ver == version:
-                    return view
-                del _ops._stripped_views[i]
-                break
-    stripped = cu_seqlens[1:]
-    vals = _ops.host_cu_seqlens(cu_seqlens, allow_sync=False)
-    if vals is not None:
-        _ops.remember_host_cu(stripped, vals[1:])
-    if version is not None:
-        _ops._stripped_views[:] = [e for e in _ops._stripped_views if e[0]() is not None][-3:]
-        _ops._stripped_views.append((weakref.ref(cu_seqlens), version, stripped))
-    return stripped
+    with _ops._cache_lock:
+        if version is not None:
+            for i in range(len(_ops._stripped_views) - 1, -1, -1):
+                ref, ver, view = _ops._stripped_views[i]
+                if ref() is cu_seqlens:
+                    if ver == version:
+                        return view
+                    del _ops._stripped_views[i]
+                    break
+        stripped = cu_seqlens[1:]
+        vals = _ops.host_cu_seqlens(cu_seqlens, allow_sync=False)
+        if vals is not None:
+            _ops.remember_host_cu(stripped, vals[1:])
+        if version is not None:
+            _ops._stripped_views[:] = [e for e in _ops._stripped_views if e[0]() is not None][-3:]
+            _ops._stripped_views.append((weakref.ref(cu_seqlens), version, stripped))
+        return stripped
 
 
 class StickBreakingAttention(torch.autograd.Function):

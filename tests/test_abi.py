@@ -341,3 +341,40 @@ def test_launch_bounds_cover_every_split_into_documents():
                 assert n_kv <= g.dkdv_main_tiles           # one kernel takes both groups
             else:
                 assert n_long <= g.dkdv_main_tiles and n_tail <= g.dkdv_tail_tiles
+
+
+def test_scratch_tables_grow_instead_of_multiplying(monkeypatch):
+    """Packed-document training changes the exact table size with every batch: the gradient table is one
+    buffer per (device, stream, role) that only grows, not one allocation per size."""
+    from types import SimpleNamespace
+    from stickbreaking_attention import _ops
+    monkeypatch.setattr(torch.cuda, "current_stream", lambda device=None: SimpleNamespace(cuda_stream=0))
+    monkeypatch.setattr(torch.cuda, "is_current_stream_capturing", lambda: False)
+    _ops.release_workspaces()
+    allocations = []
+    real_empty = torch.empty
+
+    def counting_empty(*a, **kw):
+        t = real_empty(*a, **kw)
+        allocations.append(t.numel())
+        return t
+    monkeypatch.setattr(torch, "empty", counting_empty)
+    import random
+    rng = random.Random(3)
+    base = 32 * 90_000     # floats; sizes wander within +-12 % as document lengths change
+    ptrs = set()
+    for _ in range(20):
+        n = int(base * rng.uniform(0.88, 1.12)) // 32 * 32
+        t = _ops._scratch_table(n, torch.device("cpu"), "grad")
+        assert t.numel() == n and t.data_ptr() % 16 == 0
+        ptrs.add(t.data_ptr())
+    assert len(allocations) <= 2 and len(ptrs) <= 2, allocations
+    assert len(_ops._gtab_cache) == 1
+    # another role (the rebuilt stick table) has a buffer of its own; a much larger request replaces, not adds
+    _ops._scratch_table(1000, torch.device("cpu"), "stick")
+    big = _ops._scratch_table(4 * base, torch.device("cpu"), "grad")
+    assert big.numel() == 4 * base and len(_ops._gtab_cache) == 2
+    held = sum(b.numel() for b in _ops._gtab_cache.values())
+    assert held <= int(4 * base * 1.13) + (1 << 17)
+    _ops.release_workspaces()
+    assert not _ops._gtab_cache

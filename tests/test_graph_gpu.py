@@ -65,3 +65,46 @@ def test_forward_and_backward_replay_from_a_hip_graph(fused):
         for name, a, b in zip(("o", "rem", "dq", "dk", "dv"), captured, eager):
             assert torch.equal(a, b), f"replay with seed {seed}: {name} differs from the eager launch"
     del junk
+
+
+def test_capture_with_a_cu_seqlens_tensor_never_seen_in_eager_mode():
+    """Under capture nothing may be read back from the device: a cu_seqlens tensor whose values the
+    Python layer does not know yet is taken as is (tables sized from max_seqlens, checks on the
+    device), and the replays still equal eager launches."""
+    from stickbreaking_attention import _ops, sb_attn_varlen
+    lengths = [260, 31, 129, 500]
+    H, T, d = 2, sum(lengths), 64
+    inv_temp = d ** -0.5
+
+    def make_cu():
+        return torch.tensor([0] + lengths, dtype=torch.int64).cumsum(0).to(torch.int32).to(DEV)
+
+    def launch(q, k, v, do, cu):
+        qg, kg, vg = (t.detach().requires_grad_() for t in (q, k, v))
+        o, rem = sb_attn_varlen(qg, kg, vg, cu, max(lengths), inv_temp, zero_start=True)
+        return (o, rem) + torch.autograd.grad(o, (qg, kg, vg), do)
+
+    static = [t.to(DEV) for t in orc.make_inputs((H, T, d), 200)]
+    warm_cu = make_cu()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        launch(*static, warm_cu)              # loads the library; this tensor object is not the captured one
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    _ops.release_workspaces()
+    fresh_cu = make_cu()                      # never passed to the library before the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = launch(*static, fresh_cu)
+    for seed in (201, 202):
+        fresh = [t.to(DEV) for t in orc.make_inputs((H, T, d), seed)]
+        for dst, src in zip(static, fresh):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = launch(*fresh, make_cu())
+        torch.cuda.synchronize()
+        for name, a, b in zip(("o", "rem", "dq", "dk", "dv"), captured, eager):
+            assert torch.equal(a, b), f"replay with seed {seed}: {name} differs from the eager launch"

@@ -34,10 +34,17 @@ def _forward_pair(lengths, H, d, seed):
     o_a, rem_a = torch.full_like(q, 7.0), torch.full_like(q[..., 0], 7.0)
     o_b, rem_b = torch.full_like(q, -3.0), torch.full_like(q[..., 0], -3.0)
     sched = torch.empty(lib.sba_schedule_bytes(ctypes.byref(prob)), dtype=torch.uint8, device=dev)
+    # one call first: the library looks its array's device address up on the first call per device
+    nat.check(lib.sba_varlen_fwd_static(ctypes.byref(prob), *views(o_a, rem_a), stream), "sba_varlen_fwd_static")
+    torch.cuda.synchronize()
+    o_a.fill_(7.0); rem_a.fill_(7.0)
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated(dev)
+    free_before = torch.cuda.mem_get_info(dev)[0]      # the driver's own count: sees a hipMalloc inside the library too
     nat.check(lib.sba_varlen_fwd_static(ctypes.byref(prob), *views(o_a, rem_a), stream), "sba_varlen_fwd_static")
+    torch.cuda.synchronize()
     assert torch.cuda.memory_allocated(dev) == before
+    assert torch.cuda.mem_get_info(dev)[0] == free_before, "sba_varlen_fwd_static changed the device's free memory"
     nat.check(lib.sba_build_schedule(ctypes.byref(prob), sched.data_ptr(), sched.numel(), stream), "sba_build_schedule")
     nat.check(lib.sba_varlen_fwd(ctypes.byref(prob), sched.data_ptr(), sched.numel(), *views(o_b, rem_b), None, 0, stream), "sba_varlen_fwd")
     torch.cuda.synchronize()
