@@ -24,14 +24,18 @@ for p in (ROOT, os.path.join(ROOT, "stickbreaking-attention_amd")):
 PEAK_BF16_TFLOPS = 2500.0   # MI355X published dense bf16 MFMA peak
 PEAK_HBM_GBS = 8000.0       # MI355X published HBM3E bandwidth
 
-# HBM bytes per launch on workload c3, from two `rocprofv3 --pmc` runs of this script
-# (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, summed over XCDs), each scaled by what the
-# same counter reads for the 256 MiB device copy of --calibrate-copy (FETCH_SIZE x2.0,
-# WRITE_SIZE x1.0).  Counters cannot be read from inside the process, so these are recorded
-# constants, valid for the library version they were measured with (profiles/c3_hbm_traffic_pmc.txt):
-# any other version of libsba.so reports null.
-MEASURED_TRAFFIC = {"sba_version": 205,
-                    "c3": {"fwd_kernel": 1.111e9, "bwd_dq_kernel": 1.075e9, "bwd_dkdv_kernel": 1.202e9}}
+# Figures that only rocprofv3 can see, on workload c3, recorded from the runs whose summaries are under profiles/
+# and valid for the library version they were measured with (any other version of libsba.so reports null).
+#   traffic: HBM bytes per launch from two `--pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per
+#     dispatch, summed over XCDs), each scaled by what the same counter reads for the 256 MiB device copy of
+#     --calibrate-copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0): profiles/c3_hbm_traffic_pmc.txt
+#   mfma_busy, valu_busy, coexec: fractions of the launch's SIMD-cycles in which the matrix pipe is busy
+#     (SQ_VALU_MFMA_BUSY_CYCLES), a vector instruction is active (4 x SQ_ACTIVE_INST_VALU) and both at once
+#     (SQ_VALU_MFMA_COEXEC_CYCLES), over 1024 SIMDs x GRBM_GUI_ACTIVE / 8: profiles/c3_sq_counters_pmc.txt
+MEASURED = {"sba_version": 207,
+            "c3": {"fwd_kernel": {"traffic": 1.093e9, "mfma_busy": 0.461, "valu_busy": 0.552, "coexec": 0.193},
+                   "bwd_dq_kernel": {"traffic": 1.107e9, "mfma_busy": 0.425, "valu_busy": 0.573, "coexec": 0.165},
+                   "bwd_dkdv_kernel": {"traffic": 1.203e9, "mfma_busy": 0.410, "valu_busy": 0.489, "coexec": 0.173}}}
 
 KERNELS = ["fwd_kernel", "bwd_dq_kernel", "bwd_dkdv_kernel"]
 
@@ -221,18 +225,20 @@ def roofline(m, lib):
     q,k,v,dO in and dk,dv out (6 N)."""
     d, pairs, kern_ms = m["d"], m["pairs"], m["kern_ms"]
     dom = max(range(3), key=lambda i: kern_ms[i])
-    traffic = None
-    if lib.sba_version() == MEASURED_TRAFFIC["sba_version"]:
-        traffic = MEASURED_TRAFFIC.get(m["name"], {}).get(KERNELS[dom])
+    seen = {"traffic": None, "mfma_busy": None, "valu_busy": None, "coexec": None}
+    if lib.sba_version() == MEASURED["sba_version"]:
+        seen.update(MEASURED.get(m["name"], {}).get(KERNELS[dom], {}))
+    traffic = seen["traffic"]
+    counters = {k: seen[k] for k in ("mfma_busy", "valu_busy", "coexec")}
     if m["cfg"]["bound"] == "hbm":
         alg = [4.0, 5.0, 6.0][dom] * m["tensor_bytes"]
         achieved = alg / (kern_ms[dom] * 1e-3) / 1e9
         return {"bound": "hbm", "kernel": KERNELS[dom], "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": achieved / PEAK_HBM_GBS, "traffic": traffic}
+                "frac": achieved / PEAK_HBM_GBS, "traffic": traffic, **counters}
     alg = [4.0, 6.0, 4.0][dom] * d * pairs
     achieved = alg / (kern_ms[dom] * 1e-3) / 1e12
     return {"bound": "mfma", "kernel": KERNELS[dom], "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-            "frac": achieved / PEAK_BF16_TFLOPS, "traffic": traffic}
+            "frac": achieved / PEAK_BF16_TFLOPS, "traffic": traffic, **counters}
 
 
 def describe(m):
@@ -307,7 +313,7 @@ def main():
         "kernel_ms": dict(zip(KERNELS, m["kern_ms"])),
         "kernel_executed_tflops": {n: (executed[i] / (m["kern_ms"][i] * 1e-3) / 1e12 if m["kern_ms"][i] > 0 else 0.0)
                                    for i, n in enumerate(KERNELS)},
-        "roofline": roofline(m, lib) if _ops.PRODUCT_SPACE else dict(roofline(m, lib), traffic=None),
+        "roofline": roofline(m, lib) if _ops.PRODUCT_SPACE else dict(roofline(m, lib), traffic=None, mfma_busy=None, valu_busy=None, coexec=None),
         "device": {"name": props.name, "cus": props.multi_processor_count, "clock_mhz": device_clock_mhz(torch),
                    "sba_version": lib.sba_version()},
     }
