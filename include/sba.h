@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define SBA_VERSION 207
+#define SBA_VERSION 208
 
 /* error codes (negative returns) */
 #define SBA_E_NULL      (-1)  /* a required pointer is NULL                         */
@@ -120,8 +120,13 @@ size_t sba_schedule_bytes(const sba_problem* p);
 /* Bytes of ONE carry table.  A table holds, per head and per document of length L, one fp32 for
  * every (32-key block, query row at or below it) pair -- about L*L/64, L rounded up to a
  * multiple of 32 so that every block starts on a 128-byte line -- plus one per row (the
- * forward leaves rem there in fp32, the backward the complete gradient of rem).  The forward
- * fills `stick_table`; the backward additionally needs a `grad_table` of the same size.
+ * forward leaves rem there in fp32, the backward the complete gradient of rem) -- and, behind
+ * all heads, 256 bytes of work counters: the dk/dv pass of a large problem is launched with one
+ * workgroup per compute unit, and those workgroups draw their key tiles from counters kept at
+ * the end of `grad_table` (cleared by the dq pass that precedes them; both sizes below include
+ * the 256 bytes).  The forward fills `stick_table`; the backward additionally needs a
+ * `grad_table` of the same size, which must not be shared by backward calls that run at the
+ * same time.
  *   sba_table_bytes              no lengths needed: the most any documents of at most
  *                                max_doc_len tokens can need (exact for the fixed-length op);
  *   sba_table_bytes_for_lengths  exact, from the document lengths in HOST memory.
@@ -261,6 +266,15 @@ const char* sba_error_string(int code);
  * sba_varlen_fwd_static ignores it. */
 void  sba_set_timing(int on);
 float sba_last_kernel_ms(int which);
+
+/* Test and tuning switch (no counterpart upstream, process-wide like the one above): the number of
+ * workgroups the main kernel of the dk/dv pass is launched with when it has more key tiles
+ * (times heads) than that to work through.  n > 0: exactly n rounded down to a multiple of 8 (at
+ * least 8), however few tiles there are per workgroup; n = 0 (default): one per compute unit,
+ * and only for problems with at least eight tiles per workgroup; n < 0: always one workgroup per
+ * tile.  The results do not depend on it (every tile is computed by the same instructions in the
+ * same order whichever workgroup takes it). */
+void  sba_set_dkdv_workgroups(int n);
 
 #ifdef __cplusplus
 }

@@ -16,6 +16,7 @@ using namespace sba;
 
 // Process-wide on purpose: PyTorch runs the backward on its own autograd thread.
 std::atomic<int> g_timing{0};
+std::atomic<int> g_dkdv_workgroups{0};   // sba_set_dkdv_workgroups
 std::atomic<float> g_ms[3];
 
 inline int cdiv_i(long long a, long long b) { return (int)((a + b - 1) / b); }
@@ -109,6 +110,22 @@ View to_view(const sba_view* v) {
   return r;
 }
 
+// The counter words at the end of a table workspace of `table_bytes` bytes.
+unsigned* work_words(float* table, size_t table_bytes) {
+  return reinterpret_cast<unsigned*>(table) + (table_bytes / sizeof(unsigned) - WORK_WORDS);
+}
+
+// Compute units of the current device (0 if it cannot be asked: launches then take one workgroup per item).
+int device_cus() {
+  static std::atomic<int> cached[64];   // by device ordinal; 0 = not asked yet
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if ((n = cached[dev].load(std::memory_order_relaxed)) > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+  cached[dev].store(n, std::memory_order_relaxed);
+  return n;
+}
+
 int check_arch() {
   static int cached = -1;   // immutable once set
   if (cached >= 0) return cached ? 0 : SBA_E_ARCH;
@@ -160,6 +177,9 @@ int fill_common(const sba_problem* p, bool fixed, const Sizes& sz, const void* s
   if (sched_bytes < schedule_bytes(sz)) return SBA_E_WORKSPACE;
   a->tab_stride = -1;
   if (with_table) {
+    // (the last WORK_WORDS words of a table workspace are the work counters of the call's persistent launches)
+    if (table_bytes < WORK_WORDS * sizeof(unsigned)) return SBA_E_WORKSPACE;
+    table_bytes -= WORK_WORDS * sizeof(unsigned);
     a->tab_stride = (int64_t)(table_bytes / sizeof(float) / (size_t)p->heads) & ~(int64_t)31;   // heads start on 128-byte lines
     // fixed-length needs are known here; packed documents are checked on the device against
     // what the scheduler found (kernels refuse to run, outputs are filled with NaN)
@@ -233,6 +253,14 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, size_t sche
   a.dq = to_view(dq); a.dk = to_view(dk); a.dv = to_view(dv);
   a.stick = const_cast<float*>(stick);
   a.gtab = gtab;
+  // The main kernel of the dk/dv pass fills a compute unit with one workgroup.  With many more key tiles than
+  // compute units it is launched once per compute unit and walks the tiles itself (see work_next in
+  // sba_device.hpp); with few it pays more for the hand-over between tiles than the hardware does for a
+  // fresh workgroup (measured: 960 tiles on 256 compute units, 124 against 118 us).
+  const int forced = g_dkdv_workgroups.load();
+  a.work = work_words(gtab, table_bytes);
+  a.resident = forced > 0 ? forced : (forced < 0 ? 0 : device_cus());
+  a.min_items_each = forced > 0 ? 1 : 8;
   a.max_doc_len = declared_max_doc_len(p, fixed);
   const BwdBounds bb = backward_bounds(p, fixed, sz);
   const int n_long_max = bb.n_long_max, n_tail_max = bb.n_tail_max;
@@ -308,7 +336,7 @@ size_t sba_table_bytes(const sba_problem* p) {
   Sizes sz;
   const bool fixed = p != nullptr && (p->flags & SBA_FIXED_LENGTH) != 0;
   if (check_problem(p, fixed, &sz)) return 0;
-  return (size_t)p->heads * (size_t)table_entries_bound(p, fixed) * sizeof(float);
+  return (size_t)p->heads * (size_t)table_entries_bound(p, fixed) * sizeof(float) + WORK_WORDS * sizeof(unsigned);
 }
 
 size_t sba_table_bytes_for_lengths(const sba_problem* p, const int64_t* doc_lengths, int n_lengths) {
@@ -322,7 +350,8 @@ size_t sba_table_bytes_for_lengths(const sba_problem* p, const int64_t* doc_leng
     entries += tab_doc_entries((int)doc_lengths[i]);
   }
   if (entries > 0x7fffffffll) return 0;   // a document's base must fit the scheduler's int32 field
-  return (size_t)p->heads * (size_t)(entries > 0 ? entries : 32) * sizeof(float);   // never empty: one 128-byte line per head
+  return (size_t)p->heads * (size_t)(entries > 0 ? entries : 32) * sizeof(float)   // never empty: one 128-byte line per head
+         + WORK_WORDS * sizeof(unsigned);
 }
 
 int sba_build_schedule(const sba_problem* p, void* schedule, size_t schedule_size, void* stream) {
@@ -430,6 +459,7 @@ int sba_launch_geometry(const sba_problem* p, sba_geometry* out) {
 }
 
 void sba_set_timing(int on) { g_timing.store(on); }
+void sba_set_dkdv_workgroups(int n) { g_dkdv_workgroups.store(n); }
 float sba_last_kernel_ms(int which) {
   if (which < 0 || which >= 3) return 0.f;
   std::lock_guard<std::mutex> lock(g_ev_mutex);

@@ -122,6 +122,8 @@ __global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
   const Tile t = reinterpret_cast<const Tile*>(sched + SCHED_HDR)[slot];
   asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch), "s"(t.tab_base));   // keep the tile read above the branch
   const bool refused = hdr.x != 0 || hdr.w > a.tab_stride || sched[SCHED_MAXLEN] > a.max_doc_len;
+  // the dk/dv pass that follows on the same stream hands out its work items through these counters
+  if (a.work != nullptr && blockIdx.x == 0 && threadIdx.x < WORK_WORDS) a.work[threadIdx.x] = 0u;
   if (refused || slot >= hdr.y) {
     if (a.clear_spare) {     // for the dk/dv pass as well, which has no slots to spare
       int row0, row1;
@@ -356,20 +358,30 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   // p and dz staged [query][key]: 16-byte row writes, transpose reads.
   __shared__ __attribute__((aligned(16))) unsigned short Ps[2 * PTILE];
   __shared__ __attribute__((aligned(16))) unsigned short Zs[2 * PTILE];
+  __shared__ int mbox[2][8];        // persistent launch, by item parity: the tile descriptor of the item after the current one
+                                    // (five words) and, in word 7, that item (-1: none)
 
-  // Header words and this workgroup's tile are fetched together (the grid never exceeds the
-  // allocated list, so the tile read is safe before the count is known): one round trip.
+  // A work item is one key tile of one head: item = slot * heads + head, the number blockIdx.x has
+  // when the launch takes one workgroup per item.  Header words and the first item's tile are
+  // fetched together (the grid never exceeds the allocated list, so the tile read is safe before
+  // the count is known): one round trip.
   const int* sched = a.sched;
-  const int slot = blockIdx.x / a.heads;
-  const int head = blockIdx.x - slot * a.heads;
+  const Tile* const kv_list = reinterpret_cast<const Tile*>(sched + a.kv_list_off);
   const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, table entries needed
-  const Tile t = reinterpret_cast<const Tile*>(sched + a.kv_list_off)[slot];
-  asm volatile("" ::"s"(t.tok_start), "s"(t.doc_len), "s"(t.idx), "s"(t.batch), "s"(t.tab_base));   // keep the tile read above the branch
+  const Tile t_first = kv_list[blockIdx.x / a.heads];
+  asm volatile("" ::"s"(t_first.tok_start), "s"(t_first.doc_len), "s"(t_first.idx), "s"(t_first.batch), "s"(t_first.tab_base));   // keep the tile read above the branch
   // with a kernel of their own for the documents' last key tiles, this one stops where they begin
   const int2 hdr2 = *reinterpret_cast<const int2*>(sched + SCHED_MAXLEN);   // longest document, key tiles of the first group
   const int n_mine = TailKernel<D>::value ? hdr2.y : hdr.z;
-  if (hdr.x != 0 || slot >= n_mine || hdr.w > a.tab_stride || hdr2.x > a.max_doc_len) return;
-  const int kt = t.idx;
+  const int n_items = n_mine * a.heads;
+  if (hdr.x != 0 || (int)blockIdx.x >= n_items || hdr.w > a.tab_stride || hdr2.x > a.max_doc_len) return;
+  // Persistent launch (see work_next): fewer workgroups than items; every workgroup goes on to further
+  // items, and the end of one item (last products, conversion and stores of dk / dv by the product waves)
+  // overlaps the beginning of the next (tile descriptor, K / V fragments, first Q / dO tiles and table rows,
+  // all requested by the score waves, which have nothing else to do by then).
+  const bool persistent = a.work != nullptr && (int)gridDim.x < a.n_items;   // (uniform)
+  unsigned* const ctr = a.work + WORK_DKDV;
+  const int cls = blockIdx.x & 7;
 
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -379,19 +391,46 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   // (Pairing the score waves on two SIMDs and the product waves on the other two was measured: 1.10 against 0.97 ms.)
   const bool scorer = w < 4;
   const int rw = w & 3;                              // index of the wave inside its role
+  const int ptid = rw * 64 + lane;                   // index of the thread inside its role
 
-  const int64_t tok0 = t.tok_start;
-  const elem_t* qb = reinterpret_cast<const elem_t*>(a.q.ptr) + t.batch * a.q.sb + head * a.q.sh + tok0 * a.q.st;
-  const elem_t* kb = reinterpret_cast<const elem_t*>(a.k.ptr) + t.batch * a.k.sb + head * a.k.sh + tok0 * a.k.st;
-  const elem_t* vb = reinterpret_cast<const elem_t*>(a.v.ptr) + t.batch * a.v.sb + head * a.v.sh + tok0 * a.v.st;
-  const elem_t* gob = reinterpret_cast<const elem_t*>(a.go.ptr) + t.batch * a.go.sb + head * a.go.sh + tok0 * a.go.st;
-  const Rows qrows = make_rows(qb, a.q.st, t.doc_len);
-  const Rows grows = make_rows(gob, a.go.st, t.doc_len);
-  const Rows krows = make_rows(kb, a.k.st, t.doc_len);
-  const Rows vrows = make_rows(vb, a.v.st, t.doc_len);
-
-  const int q_first = kt * BKV;                                  // first query that can see the tile
-  const int nsteps = (t.doc_len - q_first + BQ - 1) / BQ;        // >= 1
+  // What identifies an item (all uniform); each role derives the rest where it needs it.
+  struct Item { int tok_start, doc_len, kt, batch, tab_base, head; };
+  auto describe = [&](int item, const Tile& t) {
+    const int slot = item / a.heads;
+    Item it;
+    it.tok_start = t.tok_start; it.doc_len = t.doc_len; it.kt = t.idx; it.batch = t.batch; it.tab_base = t.tab_base;
+    it.head = item - slot * a.heads;
+    return it;
+  };
+  auto rows_of = [](const View& v, const Item& it) {
+    return make_rows(reinterpret_cast<const elem_t*>(v.ptr) + it.batch * v.sb + it.head * v.sh + (int64_t)it.tok_start * v.st,
+                     v.st, it.doc_len);
+  };
+  Item cur = describe(blockIdx.x, t_first);
+  // The item after the current one and its tile descriptor, as the first score wave left them in `mbox` (every wave,
+  // behind the barrier of the current item's last step).
+  auto next_item = [&](int parity, Item& it) {
+    if (!persistent) return -1;
+    const int nx = __builtin_amdgcn_readfirstlane(mbox[parity][7]);
+    if (nx < 0) return -1;
+    Tile t;
+    t.tok_start = __builtin_amdgcn_readfirstlane(mbox[parity][0]);
+    t.doc_len = __builtin_amdgcn_readfirstlane(mbox[parity][1]);
+    t.idx = __builtin_amdgcn_readfirstlane(mbox[parity][2]);
+    t.batch = __builtin_amdgcn_readfirstlane(mbox[parity][3]);
+    t.tab_base = __builtin_amdgcn_readfirstlane(mbox[parity][4]);
+    it = describe(nx, t);
+    return nx;
+  };
+  // Both roles copy Q / dO tiles into the ring.  The product waves copy every tile from tile AHEAD on, AHEAD steps
+  // ahead of its use, and the first AHEAD tiles of a workgroup's first item; the score waves copy the first AHEAD
+  // tiles of every later item, at a time when the product waves are still busy with the item before.
+  // (a 32 x 32 tile is one instruction each for two waves: the other two request nothing, wait
+  // for nothing and meet the copies at the barrier)
+  constexpr int CT = D == 32 ? NPT / 2 : NPT;   // threads of a role that copy tiles
+  const bool copier = ptid < CT;                // (uniform per wave)
+  using Copy = TileCopy<D, BQ, CT, false>;
+  constexpr int LOADS_PER_TILE = 2 * Copy::NCH;
 
   // The two roles run separate copies of the step loop (same barrier count) so that neither
   // carries the other's registers.
@@ -401,38 +440,12 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
   if (scorer) {
     __builtin_amdgcn_s_setprio(3);
     const int sb = rw;                          // 32-key block of this wave
-    const int k0 = kt * BKV + 32 * sb;
     const int qr = n;                           // this lane's query row inside a tile
     el8 kf[KS], vf[KS];                      // MFMA row n holds key k0 + kperm(n)
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      kf[ks] = load_frag(krows, k0 + kperm(n), 32 * ks + 16 * h);
-      vf[ks] = load_frag(vrows, k0 + kperm(n), 32 * ks + 16 * h);
-    }
-    // A block that starts past the end of the document is never visible to a query; its table
-    // reads are redirected to the document's last block so that they stay inside the document's
-    // table area, and their values are never used.  (Rows above a block's first row, read by the
-    // first steps of the later blocks, fall into the preceding block's rows: in bounds, unused.)
-    const int tblock = min((BKV / 32) * kt + sb, (t.doc_len - 1) / 32);
-    const int64_t tab_row0 = (int64_t)head * a.tab_stride + t.tab_base;
-    const int64_t tab = tab_row0 + tab_seg32(t.doc_len, tblock);
-    const int64_t tab_rowval = tab_row0 + tab_rowplane32(t.doc_len);   // per-row plane: rem (stick table), d(rem) (gradient table, written by the dq pass)
-    // Fused output o + rem * v: its gradient reaches v_j directly as rem_j * do_j.  The queries of
-    // step `sb` are this wave's own keys, so that term is dv = P^T dO with rem_j added on the
-    // diagonal of P (which is otherwise zero, or p_jj with attend_current), at no extra traffic.
-    float rem_own = 0.0f;
-    if (a.fuse && k0 + n < t.doc_len) rem_own = a.stick[tab_rowval + k0 + n];
-    // Per-row carries of a step.  The three runs of rows this wave reads (its block's rows of the two
-    // tables and the per-row plane of the gradient table) are buffer resources, so that a lane
-    // addresses them with a 32-bit byte offset: two vector instructions per step instead of 64-bit
-    // address arithmetic per load.  The row is clamped into the document; rows past its end then
-    // carry the values of its last row, which is harmless: their Q and dO rows are zero (the tile
-    // copies fill them with zeros), so whatever finite p and dz they produce adds nothing to dk, dv.
-    const unsigned run_bytes = (unsigned)t.doc_len * 4u;   // (rows of one block: at most doc_len)
-    const __amdgpu_buffer_rsrc_t stick_rs = __builtin_amdgcn_make_buffer_rsrc(a.stick + tab, 0, run_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t gtab_rs = __builtin_amdgcn_make_buffer_rsrc(a.gtab + tab, 0, run_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t drem_rs = __builtin_amdgcn_make_buffer_rsrc(a.gtab + tab_rowval, 0, run_bytes, 0x00020000);
-    const int row4 = 4 * (q_first + qr), last4 = 4 * (t.doc_len - 1);
+    // of the current item
+    int k0, q_first, nsteps, doc_len, row4, last4;
+    float rem_own;
+    __amdgpu_buffer_rsrc_t stick_rs, gtab_rs, drem_rs;
     // `request` only issues the loads; nothing consumes (and therefore waits for) a loaded value
     // until `settle`, a whole step or more after the request.
     struct Raw { float e, g, d; };
@@ -447,6 +460,76 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       ce = r.e;
       cc = r.g;
       d_r = r.d;
+    };
+    // work queue of a persistent launch (see `queue` below)
+    unsigned ticket = 0;
+    int tile_word = -1;
+    const bool keeper = persistent && rw == 0;     // (uniform)
+    int queue_from = 0x7fffffff;                   // of the current item: the step of the draw (never, for the other waves)
+    Raw r0, r1, r2;
+    // Everything of an item that comes from global memory, requested in one go: the first AHEAD Q / dO
+    // tiles, the K and V fragments of this wave's keys and the carries of the first three steps.  For
+    // every item but a workgroup's first this happens right after the score waves' last step of the
+    // item before, while the product waves finish that one.
+    auto open_item = [&](const KArgs& a, const Item& it, bool with_tiles) {
+      // (Inside the item loop the argument block is read afresh, see the call, and the lane indices are opaque
+      // here: the views and the per-lane address parts would otherwise be formed once, ahead of the item loop,
+      // and held in registers all through the steps, which have none to spare.)
+      int n = lane & 31, h = lane >> 5;
+      asm volatile("" : "+v"(n), "+v"(h));
+      doc_len = it.doc_len;
+      q_first = it.kt * BKV;                                  // first query that can see the tile
+      k0 = q_first + 32 * sb;
+      nsteps = (doc_len - q_first + BQ - 1) / BQ;             // >= 1
+      // A block that starts past the end of the document is never visible to a query; its table
+      // reads are redirected to the document's last block so that they stay inside the document's
+      // table area, and their values are never used.  (Rows above a block's first row, read by the
+      // first steps of the later blocks, fall into the preceding block's rows: in bounds, unused.)
+      const int tblock = min((BKV / 32) * it.kt + sb, (doc_len - 1) / 32);
+      const int64_t tab_row0 = (int64_t)it.head * a.tab_stride + it.tab_base;
+      const int64_t tab = tab_row0 + tab_seg32(doc_len, tblock);
+      const int64_t tab_rowval = tab_row0 + tab_rowplane32(doc_len);   // per-row plane: rem (stick table), d(rem) (gradient table, written by the dq pass)
+      // Fused output o + rem * v: its gradient reaches v_j directly as rem_j * do_j.  The queries of
+      // step `sb` are this wave's own keys, so that term is dv = P^T dO with rem_j added on the
+      // diagonal of P (which is otherwise zero, or p_jj with attend_current), at no extra traffic.
+      rem_own = 0.0f;
+      if (a.fuse && k0 + n < doc_len) rem_own = a.stick[tab_rowval + k0 + n];
+      // Per-row carries of a step.  The three runs of rows this wave reads (its block's rows of the two
+      // tables and the per-row plane of the gradient table) are buffer resources, so that a lane
+      // addresses them with a 32-bit byte offset: two vector instructions per step instead of 64-bit
+      // address arithmetic per load.  The row is clamped into the document; rows past its end then
+      // carry the values of its last row, which is harmless: their Q and dO rows are zero (the tile
+      // copies fill them with zeros), so whatever finite p and dz they produce adds nothing to dk, dv.
+      const unsigned run_bytes = (unsigned)doc_len * 4u;   // (rows of one block: at most doc_len)
+      stick_rs = __builtin_amdgcn_make_buffer_rsrc(a.stick + tab, 0, run_bytes, 0x00020000);
+      gtab_rs = __builtin_amdgcn_make_buffer_rsrc(a.gtab + tab, 0, run_bytes, 0x00020000);
+      drem_rs = __builtin_amdgcn_make_buffer_rsrc(a.gtab + tab_rowval, 0, run_bytes, 0x00020000);
+      row4 = 4 * (q_first + qr);
+      last4 = 4 * (doc_len - 1);
+      if (copier && with_tiles) {
+        const Rows qrows = rows_of(a.q, it), grows = rows_of(a.go, it);
+        Copy qcopy, gcopy;      // (formed here, once per item: a score wave has no register to keep them in)
+        qcopy.init(64 * rw + 32 * h + n, qrows.row_bytes);
+        gcopy.init(64 * rw + 32 * h + n, grows.row_bytes);
+#pragma unroll
+        for (int sft = 0; sft < AHEAD; ++sft)
+          if (sft < nsteps) {
+            qcopy.issue(qrows, q_first + sft * BQ, Qs + sft * QTILE);
+            gcopy.issue(grows, q_first + sft * BQ, Gs + sft * QTILE);
+          }
+      }
+      {
+        const Rows krows = rows_of(a.k, it), vrows = rows_of(a.v, it);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          kf[ks] = load_frag(krows, k0 + kperm(n), 32 * ks + 16 * h);
+          vf[ks] = load_frag(vrows, k0 + kperm(n), 32 * ks + 16 * h);
+        }
+      }
+      request(0, r0);
+      request(1, r1);
+      request(2, r2);
+      if (keeper) queue_from = max(nsteps - 5, 0);
     };
     // The row-read offsets of this lane inside a tile (chunk 2*ks + h of row qr).
     int roff[KS];
@@ -482,11 +565,6 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     // Carries are requested three steps before the step that uses them, into three register sets
     // used in turn (a table read takes longer than one step), and settled when that step begins.
     float carry_e, carry_c, dr;
-    Raw r0, r1, r2;
-    request(0, r0);
-    request(1, r1);
-    request(2, r2);
-    lds_barrier();                        // tiles 0 and 1 are in slots 0 and 1
     // One step: (xc, dc) hold the finished chains of block i; the chains of block i+1 go into
     // (xn, dn).  Called with the two accumulator pairs swapped on alternate steps, so nothing
     // is copied between steps.  DIAG = one of the first steps, whose queries may sit on or
@@ -619,37 +697,85 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       if constexpr (PROD && D >= 64) bulk(slot_tag, i, xc, dc, xn, dn, set);   // (its eight chunks need 2 * KS >= 8 chain steps)
       else step(std::false_type{}, i, xc, dc, xn, dn, set);
     };
-    f32x16 xa, da, xb, db;
-    chains(0, xa, da);
-    // the first BKV/BQ = 4 steps can touch the diagonal of some wave's block
-    step(std::true_type{}, 0, xa, da, xb, db, r0);
-    if (nsteps > 1) step(std::true_type{}, 1, xb, db, xa, da, r1);
-    if (nsteps > 2) step(std::true_type{}, 2, xa, da, xb, db, r2);
-    if (nsteps > 3) step(std::true_type{}, 3, xb, db, xa, da, r0);
-    // Whole turns of the ring with static slots (the ring, the two staging buffers, the two
-    // accumulator pairs and the three carry sets all repeat with period six: at i = 4 + 6m tile
-    // i+1 sits in slot 5 and the carries in set 1), then the remaining steps with run-time slots.
-    using std::integral_constant;
-    int i = BKV / BQ;
+    // Work queue of a persistent launch, kept by the first score wave ahead of the steps: the draw goes out five
+    // steps before the item ends; two steps before the end its answer is taken and the tile descriptor of the
+    // next item requested (one word per lane); ahead of the last step both go into `mbox`, where every wave finds
+    // them behind that step's barrier -- no wave ever waits for the queue or for the descriptor.  A score wave's
+    // only other global loads in a step are the three of `request`, and loads return in the order issued: "at
+    // most 3 * (steps since the draw) outstanding" says that the draw has returned.
+    auto queue = [&](int i, int parity) {
+      if (i < queue_from) return;                  // (all a step away from the item's end pays for the queue: one comparison)
+      const int drawn = queue_from, resolved = max(nsteps - 2, 0);
+      if (i == drawn && lane == 0) ticket = work_draw(ctr + cls);
+      if (i == resolved) {
+        const int since = resolved - drawn;
+        if (since >= 3) wait_loads<9>();
+        else if (since == 2) wait_loads<6>();
+        else if (since == 1) wait_loads<3>();
+        else wait_loads<0>();
+        int nx = -1;
+        if (lane == 0) {
+          work_wait(ticket);     // (nothing left to wait for: ties the value to the waits above)
+          nx = work_next(ctr, cls, ticket, n_items, gridDim.x);
+        }
+        nx = __builtin_amdgcn_readfirstlane(nx);
+        tile_word = nx;
+        if (nx >= 0 && lane < 7) tile_word = reinterpret_cast<const int*>(kv_list + nx / a.heads)[lane];
+      }
+      if (i == nsteps - 1 && lane < 8) mbox[parity][lane] = tile_word;
+    };
+    open_item(a, cur, false);     // (a workgroup's first item: the product waves, idle so far, copy its first tiles)
 #pragma unroll 1
-    for (; i + RING <= nsteps; i += RING) {
-      later(integral_constant<int, 5>{}, i, xa, da, xb, db, r1);
-      later(integral_constant<int, 0>{}, i + 1, xb, db, xa, da, r2);
-      later(integral_constant<int, 1>{}, i + 2, xa, da, xb, db, r0);
-      later(integral_constant<int, 2>{}, i + 3, xb, db, xa, da, r1);
-      later(integral_constant<int, 3>{}, i + 4, xa, da, xb, db, r2);
-      later(integral_constant<int, 4>{}, i + 5, xb, db, xa, da, r0);
+    for (int m = 0;; ++m) {
+      wait_loads<9>();                      // all but the carries have arrived: tiles and fragments
+      lds_barrier();                        // every score wave's part of tiles 0 .. AHEAD-1 is in slots 0 .. AHEAD-1
+      f32x16 xa, da, xb, db;
+      chains(0, xa, da);
+      // the first BKV/BQ = 4 steps can touch the diagonal of some wave's block
+      queue(0, m & 1);
+      step(std::true_type{}, 0, xa, da, xb, db, r0);
+      if (nsteps > 1) { queue(1, m & 1); step(std::true_type{}, 1, xb, db, xa, da, r1); }
+      if (nsteps > 2) { queue(2, m & 1); step(std::true_type{}, 2, xa, da, xb, db, r2); }
+      if (nsteps > 3) { queue(3, m & 1); step(std::true_type{}, 3, xb, db, xa, da, r0); }
+      // Whole turns of the ring with static slots (the ring, the two staging buffers, the two
+      // accumulator pairs and the three carry sets all repeat with period six: at i = 4 + 6m tile
+      // i+1 sits in slot 5 and the carries in set 1), then the remaining steps with run-time slots.
+      using std::integral_constant;
+      int i = BKV / BQ;
+      // (the queue's business all falls into an item's last five steps: the turns before them run without it, as one
+      // straight-line block)
+#pragma unroll 1
+      for (; i + RING + 5 <= nsteps; i += RING) {
+        later(integral_constant<int, 5>{}, i, xa, da, xb, db, r1);
+        later(integral_constant<int, 0>{}, i + 1, xb, db, xa, da, r2);
+        later(integral_constant<int, 1>{}, i + 2, xa, da, xb, db, r0);
+        later(integral_constant<int, 2>{}, i + 3, xb, db, xa, da, r1);
+        later(integral_constant<int, 3>{}, i + 4, xa, da, xb, db, r2);
+        later(integral_constant<int, 4>{}, i + 5, xb, db, xa, da, r0);
+      }
+#pragma unroll 1
+      for (; i + RING <= nsteps; i += RING) {
+        queue(i, m & 1);     later(integral_constant<int, 5>{}, i, xa, da, xb, db, r1);
+        queue(i + 1, m & 1); later(integral_constant<int, 0>{}, i + 1, xb, db, xa, da, r2);
+        queue(i + 2, m & 1); later(integral_constant<int, 1>{}, i + 2, xa, da, xb, db, r0);
+        queue(i + 3, m & 1); later(integral_constant<int, 2>{}, i + 3, xb, db, xa, da, r1);
+        queue(i + 4, m & 1); later(integral_constant<int, 3>{}, i + 4, xa, da, xb, db, r2);
+        queue(i + 5, m & 1); later(integral_constant<int, 4>{}, i + 5, xb, db, xa, da, r0);
+      }
+      // (i = 4 + 6m here: accumulator pair a and carry set 1 are next)
+      if (i < nsteps) { queue(i, m & 1); later(integral_constant<int, -1>{}, i, xa, da, xb, db, r1); }
+      if (i + 1 < nsteps) { queue(i + 1, m & 1); later(integral_constant<int, -1>{}, i + 1, xb, db, xa, da, r2); }
+      if (i + 2 < nsteps) { queue(i + 2, m & 1); later(integral_constant<int, -1>{}, i + 2, xa, da, xb, db, r0); }
+      if (i + 3 < nsteps) { queue(i + 3, m & 1); later(integral_constant<int, -1>{}, i + 3, xb, db, xa, da, r1); }
+      if (i + 4 < nsteps) { queue(i + 4, m & 1); later(integral_constant<int, -1>{}, i + 4, xa, da, xb, db, r2); }
+      // This wave is done with the item's tiles and with its K / V fragments: the next item's global
+      // reads go out now, while the product waves form the last products and convert and store dk / dv.
+      const int next = next_item(m & 1, cur);
+      if (next < 0) break;
+      open_item(fresh_args(), cur, true);
     }
-    // (i = 4 + 6m here: accumulator pair a and carry set 1 are next)
-    if (i < nsteps) later(integral_constant<int, -1>{}, i, xa, da, xb, db, r1);
-    if (i + 1 < nsteps) later(integral_constant<int, -1>{}, i + 1, xb, db, xa, da, r2);
-    if (i + 2 < nsteps) later(integral_constant<int, -1>{}, i + 2, xa, da, xb, db, r0);
-    if (i + 3 < nsteps) later(integral_constant<int, -1>{}, i + 3, xb, db, xa, da, r1);
-    if (i + 4 < nsteps) later(integral_constant<int, -1>{}, i + 4, xa, da, xb, db, r2);
-    lds_barrier();                        // the product waves' last step
   } else {
     __builtin_amdgcn_s_setprio(0);
-    const int ptid = rw * 64 + lane;
     const int mat = (rw >> 1) & 1, half = rw & 1;   // (dv | dk) x 64 keys (two 32-key blocks); all D columns
     f32x16 acc[2][DB];
 #pragma unroll
@@ -675,27 +801,18 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
         yoff[u][j] = swz_off<D>(r, yc >> 3) + (yc & 7);
       }
     }
-    // Tile staging by the 256 product threads: asynchronous global -> LDS copies straight into
-    // the ring slot, well ahead of the score waves that will read it.
-    // (a 32 x 32 tile is one instruction each for two waves: the other two request nothing, wait
-    // for nothing and meet the copies at the barrier)
-    constexpr int CT = D == 32 ? NPT / 2 : NPT;   // threads that copy tiles
-    const bool copier = ptid < CT;                // (uniform per wave)
-    using Copy = TileCopy<D, BQ, CT, false>;
-    constexpr int LOADS_PER_TILE = 2 * Copy::NCH;
     Copy qcopy, gcopy;
-    qcopy.init(ptid, qrows.row_bytes);
-    gcopy.init(ptid, grows.row_bytes);
+    qcopy.init(ptid, (unsigned)a.q.st * 2u);
+    gcopy.init(ptid, (unsigned)a.go.st * 2u);
+    // of the current item
+    Rows qrows = rows_of(a.q, cur), grows = rows_of(a.go, cur);
+    int q_first = cur.kt * BKV;
+    int nsteps = (cur.doc_len - q_first + BQ - 1) / BQ;
     auto fetch = [&](int step) {
       if (!copier) return;
       qcopy.issue(qrows, q_first + step * BQ, Qs + (step % RING) * QTILE);
       gcopy.issue(grows, q_first + step * BQ, Gs + (step % RING) * QTILE);
     };
-#pragma unroll
-    for (int sft = 0; sft < AHEAD; ++sft)
-      if (sft < nsteps) fetch(sft);
-    wait_loads<0>();
-    lds_barrier();
     // The LDS is the busiest unit of this kernel (every step moves about 140 KB through it), and
     // a product wave that fetched all its operands after the barrier would spend half the step
     // issuing reads.  Only the staged p / dz fragments have to wait for the barrier: the Q / dO
@@ -709,10 +826,14 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     auto finish = [&](int i) {
       // Tile i+2 (read by the score waves in step i+1) has landed before anyone passes the
       // barrier: only the tiles requested after it may still be in flight (loads return in order).
-      const int after = min(i + AHEAD, nsteps - 1) - (i + 2);
-      if (after >= 2) wait_loads<2 * LOADS_PER_TILE>();
-      else if (after == 1) wait_loads<LOADS_PER_TILE>();
-      else wait_loads<0>();
+      // The first AHEAD tiles are the score waves' (landed before the item's first barrier), and the
+      // item's last two barriers guard no tile.
+      if (i + 2 >= AHEAD && i + 2 < nsteps) {
+        const int after = min(i + AHEAD, nsteps - 1) - (i + 2);
+        if (after >= 2) wait_loads<2 * LOADS_PER_TILE>();
+        else if (after == 1) wait_loads<LOADS_PER_TILE>();
+        else wait_loads<0>();
+      }
       lds_barrier();
     };
     // iteration i >= 1: products of step i - 1 with the Q / dO fragments in `cur`; the fragments of
@@ -737,25 +858,54 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
         read_y(i, nxt, ks);
         __builtin_amdgcn_sched_barrier(0);
       }
-      finish(i);
+      if (i < nsteps) finish(i);     // (nothing follows the item's last products that another wave could disturb)
     };
-    el8 ya[2][DB], yb[2][DB];
-    if (AHEAD < nsteps) fetch(AHEAD);
-    read_y(0, ya, 0);
-    read_y(0, ya, 1);
-    finish(0);
-    for (int i = 1; i <= nsteps; i += 2) {
-      iter(i, ya, yb);
-      if (i + 1 <= nsteps) iter(i + 1, yb, ya);
-    }
-    // (the last barrier of the loop has passed: the p/dz staging buffers are free)
-    const View& ov = mat ? a.dk : a.dv;
-    elem_t* outb = reinterpret_cast<elem_t*>(ov.ptr) + t.batch * ov.sb + head * ov.sh + tok0 * ov.st;
-    unsigned short* scratch = (rw & 2 ? Zs : Ps) + (rw & 1) * 32 * D;
 #pragma unroll
-    for (int kb2 = 0; kb2 < 2; ++kb2)
-      store_block32<D>(scratch, acc[kb2], mat ? a.inv_temp : 1.0f, outb, ov.st, kt * BKV + 64 * half + 32 * kb2,
-                       t.doc_len, lane);
+    for (int sft = 0; sft < AHEAD; ++sft)
+      if (sft < nsteps) fetch(sft);          // (of the workgroup's first item; the score waves copy these tiles of every later one)
+    wait_loads<0>();
+#pragma unroll 1
+    for (int m = 0;; ++m) {
+      lds_barrier();                        // the item's first barrier: tiles 0 .. AHEAD-1 are in the ring
+      el8 ya[2][DB], yb[2][DB];
+      if (AHEAD < nsteps) fetch(AHEAD);
+      read_y(0, ya, 0);
+      read_y(0, ya, 1);
+      finish(0);
+#pragma unroll 1
+      for (int i = 1; i <= nsteps; i += 2) {
+        iter(i, ya, yb);
+        if (i + 1 <= nsteps) iter(i + 1, yb, ya);
+      }
+      // dk / dv leave through ring slots 4 and 5, which nothing uses between the barrier of the item's last
+      // score step and the next item's first barrier (the score waves are filling slots 0 .. AHEAD-1 with the
+      // next item's first tiles by now; the staging buffers may still be feeding another product wave's last
+      // products).  This wave reaches that barrier only after the stores below.
+      static_assert(AHEAD + 2 <= RING, "two ring slots free for the output staging");
+      Item nxt = cur;
+      const int next = next_item(m & 1, nxt);
+      const KArgs a = fresh_args();          // (see open_item)
+      int lane_e = lane;
+      asm volatile("" : "+v"(lane_e));
+      const View& ov = mat ? a.dk : a.dv;
+      elem_t* outb = reinterpret_cast<elem_t*>(ov.ptr) + cur.batch * ov.sb + cur.head * ov.sh + (int64_t)cur.tok_start * ov.st;
+      unsigned short* scratch = (rw & 2 ? Gs : Qs) + (AHEAD + (rw & 1)) * QTILE;
+#pragma unroll
+      for (int kb2 = 0; kb2 < 2; ++kb2) {
+        store_block32<D>(scratch, acc[kb2], mat ? a.inv_temp : 1.0f, outb, ov.st, cur.kt * BKV + 64 * half + 32 * kb2,
+                         cur.doc_len, lane_e);
+#pragma unroll
+        for (int j = 0; j < DB; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[kb2][j][e] = 0.0f;
+      }
+      if (next < 0) break;
+      cur = nxt;
+      qrows = rows_of(a.q, cur);
+      grows = rows_of(a.go, cur);
+      q_first = cur.kt * BKV;
+      nsteps = (cur.doc_len - q_first + BQ - 1) / BQ;
+    }
   }
 }
 
@@ -994,12 +1144,14 @@ static hipError_t launch_dq_d(const KArgs& a, bool ac, bool prod, int n_q_max, h
 
 // n_long_max / n_last_max: upper bounds on the key tiles of the first / second group of the list.
 template <int D>
-static hipError_t launch_dkdv_d(const KArgs& a, bool ac, bool prod, int n_long_max, int n_last_max, hipStream_t s) {
+static hipError_t launch_dkdv_d(const KArgs& a_in, bool ac, bool prod, int n_long_max, int n_last_max, hipStream_t s) {
   static_assert(TailKernel<D>::value == (D <= 64), "has_dkdv_tail_kernel() states the same rule for the host");
+  KArgs a = a_in;
   const DkdvGrid g = dkdv_grid(TailKernel<D>::value, n_long_max, n_last_max, a.n_kv_alloc);
   const unsigned n_main = (unsigned)g.main_tiles;
   if (n_main > 0) {
-    const dim3 grid(n_main * (unsigned)a.heads), block(NT2);
+    a.n_items = (int)(n_main * (unsigned)a.heads);
+    const dim3 grid(launch_grid(a, a.n_items)), block(NT2);
     if (ac) {
       if (prod) hipLaunchKernelGGL((bwd_dkdv_kernel<D, true, true>), grid, block, 0, s, a);
       else hipLaunchKernelGGL((bwd_dkdv_kernel<D, true, false>), grid, block, 0, s, a);

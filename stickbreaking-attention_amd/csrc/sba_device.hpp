@@ -124,6 +124,52 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// ---------------------------------------------------------------------------------------------
+// Work queue of a persistent launch.
+//
+// The hardware deals the workgroups of a grid to the eight XCDs in turn (workgroup b runs on XCD
+// b mod 8) and each XCD then works through its share alone.  The XCDs of one part do not run at
+// the same speed (measured on the dk/dv pass: 0.875 to 1.0 us per step between the fastest and
+// the slowest XCD of one MI355X), so with one workgroup per work item the launch ends when the
+// slowest XCD is done with its eighth, the others idle for several percent of the kernel by then.
+//
+// A persistent launch therefore starts only as many workgroups as fit on the chip at once (`grid`,
+// a multiple of 8) over n_items > grid work items numbered as blockIdx used to number them.
+// Workgroup b begins with item b.  The remaining items form eight classes, item grid + c + 8 * pos
+// being position pos of class c, dealt out through one counter per class (zero when the launch
+// begins): a workgroup draws from the class of its own XCD (its items then share K/V or Q/dO rows
+// with their neighbours behind that XCD's L2 exactly as before) and, once that class is exhausted,
+// from the classes of the other XCDs.  Counters only grow and every draw either yields an item or
+// finds its class exhausted, so every workgroup ends after at most n_items + 8 draws.
+// ---------------------------------------------------------------------------------------------
+constexpr int WORK_WORDS = 64;        // counter words reserved at the end of a table workspace (256 bytes)
+constexpr int WORK_DQ = 0;            // first counter of: the forward or the dq pass,
+constexpr int WORK_DKDV = 8;          //   the dk/dv pass,
+constexpr int WORK_DKDV_TAIL = 16;    //   its kernel for the second group of key tiles
+__host__ __device__ inline int work_positions(int n_items, int grid, int c) { return (n_items - grid - c + 7) >> 3; }   // may be <= 0
+// One lane draws the next ticket of its class.  The draw goes out when the current item has only its epilogue left
+// (a draw made when the item BEGINS would hand the following item to this workgroup however long the current one
+// still takes, which is a static assignment in all but name) and is looked at after the epilogue, so its round trip
+// is hidden.  Through inline assembly: the compiler would wait for the returned value right behind the instruction.
+__device__ __forceinline__ unsigned work_draw(unsigned* ctr_of_class) {
+  unsigned ticket, zero = 0u, one = 1u;
+  asm volatile("global_atomic_add %0, %1, %2, %3 sc0" : "=&v"(ticket) : "v"(zero), "v"(one), "s"(ctr_of_class) : "memory");
+  return ticket;
+}
+__device__ __forceinline__ void work_wait(unsigned& ticket) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(ticket)::"memory"); }
+// The same lane: the item behind ticket `pos` of class `cls`, or the next item any other class still holds, or -1.
+__device__ inline int work_next(unsigned* ctr, int cls, unsigned pos, int n_items, int grid) {
+  if ((int)pos < work_positions(n_items, grid, cls)) return grid + cls + 8 * (int)pos;
+  for (int k = 1; k < 8; ++k) {
+    const int c = (cls + k) & 7;
+    const int n_pos = work_positions(n_items, grid, c);
+    if (n_pos <= 0 || (int)__hip_atomic_load(&ctr[c], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= n_pos) continue;
+    const unsigned q = atomicAdd(&ctr[c], 1u);
+    if ((int)q < n_pos) return grid + c + 8 * (int)q;
+  }
+  return -1;
+}
+
 inline namespace SBA_ELEM_NS {
 
 #ifdef SBA_ELEM_F16

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "sba_device.hpp"
 
 namespace sba {
@@ -29,7 +31,48 @@ struct KArgs {
                                // the kernels refuse to run when the scheduler found a longer one)
   float c;                     // inv_temp * log2(e)
   float inv_temp;
+  unsigned* work;              // work counters of the backward's persistent launch (WORK_WORDS words at the end of the
+                               // gradient table; the dq pass clears them), or null: one workgroup per work item
+  int n_items;                 // work items of this launch (what the grid would be with one workgroup per item)
+  int resident;                // host side: workgroups of a persistent launch (0: never persistent)
+  int min_items_each;          // host side: a launch is persistent when it has this many items per workgroup
 };
+
+// The argument block read afresh from the kernel-argument segment.  A persistent kernel calls this at
+// the top of every work item with a pointer the compiler cannot see through: argument words it
+// needs would otherwise be loaded once, ahead of the item loop, and stay in scalar registers across
+// the whole loop (the block is 380 bytes; the loop bodies have no such room, and spilled scalar
+// registers end up as vector registers spilled to scratch memory).
+__device__ __forceinline__ KArgs fresh_args() {
+  typedef const __attribute__((address_space(4))) unsigned long long* Words;
+  Words w = (Words)__builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(w));
+  static_assert(sizeof(KArgs) % 8 == 0, "copied in 8-byte words");
+  union { KArgs a; unsigned long long u[sizeof(KArgs) / 8]; } out;
+#pragma unroll
+  for (unsigned i = 0; i < sizeof(KArgs) / 8; ++i) out.u[i] = w[i];
+  // Pointers rebuilt from integer words are generic pointers to the compiler (64-bit flat addresses in
+  // vector registers for every access); say again what it knows of pointers in a kernel's argument
+  // list: they point into global memory.
+  auto global = [](auto*& p) {
+    typedef __attribute__((address_space(1))) char* GlobalBytes;
+    p = reinterpret_cast<std::remove_reference_t<decltype(p)>>((char*)(GlobalBytes)(unsigned long long)p);
+  };
+  KArgs& a = out.a;
+  global(a.q.ptr); global(a.k.ptr); global(a.v.ptr); global(a.o.ptr); global(a.rem.ptr);
+  global(a.go.ptr); global(a.grem.ptr); global(a.dq.ptr); global(a.dk.ptr); global(a.dv.ptr);
+  global(a.sched); global(a.stick); global(a.gtab); global(a.weights); global(a.work);
+  return out.a;
+}
+
+// Grid of a launch over n_items work items: one workgroup per item, or -- when the caller has work counters and
+// there are enough items for every workgroup of a persistent launch -- a.resident workgroups (a multiple of 8).
+inline unsigned launch_grid(const KArgs& a, long long n_items) {
+  const long long resident = a.resident & ~7;
+  const bool persistent = a.work != nullptr && resident >= 8 && n_items > resident &&
+                          n_items >= resident * (long long)a.min_items_each;
+  return (unsigned)(persistent ? resident : n_items);
+}
 
 struct SchedArgs {
   const void* cu;   // null for fixed-length

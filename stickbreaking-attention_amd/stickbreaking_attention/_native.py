@@ -56,7 +56,7 @@ class SbaGeometry(ctypes.Structure):
 EXPORTS = (
     "sba_version", "sba_error_string", "sba_schedule_bytes", "sba_table_bytes", "sba_table_bytes_for_lengths",
     "sba_build_schedule",
-    "sba_varlen_fwd", "sba_varlen_bwd", "sba_attn_fwd", "sba_attn_bwd", "sba_set_timing",
+    "sba_varlen_fwd", "sba_varlen_bwd", "sba_attn_fwd", "sba_attn_bwd", "sba_set_timing", "sba_set_dkdv_workgroups",
     "sba_last_kernel_ms", "sba_varlen_fwd_weights", "sba_attn_fwd_weights", "sba_varlen_fwd_static",
     "sba_launch_geometry",
 )
@@ -109,6 +109,8 @@ def load():
         lib.sba_varlen_fwd_static.argtypes = [P, V, V, V, V, V, vp]
         lib.sba_set_timing.restype = None
         lib.sba_set_timing.argtypes = [ctypes.c_int]
+        lib.sba_set_dkdv_workgroups.restype = None
+        lib.sba_set_dkdv_workgroups.argtypes = [ctypes.c_int]
         lib.sba_last_kernel_ms.restype = ctypes.c_float
         lib.sba_last_kernel_ms.argtypes = [ctypes.c_int]
         _lib = lib

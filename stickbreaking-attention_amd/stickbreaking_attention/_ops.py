@@ -53,6 +53,7 @@ SUPPORTED_HEAD_DIMS = (32, 64, 128)
 
 # Tile sizes the library's workspace formulas are built on (query tile, dk/dv key tile, table block).
 _BM, _BKV, _BT, _SCHED_HDR, _TILE_WORDS = 128, 128, 32, 16, 8
+_WORK_WORDS = 64      # words at the end of every carry table: the work counters of the library's persistent launches
 
 
 def _padded_dim(d: int) -> int:
@@ -98,7 +99,7 @@ def workspace_sizes(fixed: bool, batch: int, heads: int, tokens: int, n_docs: in
         entries = lengths if isinstance(lengths, int) else max(32, sum(table_entries(int(n)) for n in lengths))
     else:
         entries = table_entries_bound(tokens, max_doc_len, n_docs)
-    return (4 * words + 255) & ~255, heads * entries
+    return (4 * words + 255) & ~255, heads * entries + _WORK_WORDS
 
 
 # One lock for the module-level caches below (host copies of cu_seqlens, views without the leading
@@ -454,7 +455,7 @@ def check_status(sched: torch.Tensor, table: Optional[torch.Tensor] = None, head
     ``max_doc_len`` (which the backward's launch is sized with)."""
     hdr = sched[:32].view(torch.int32).tolist()
     status, need, longest = hdr[0], hdr[3], hdr[6]
-    if status == 0 and table is not None and table.numel() and need > ((table.numel() // heads) & ~31):
+    if status == 0 and table is not None and table.numel() and need > (((table.numel() - _WORK_WORDS) // heads) & ~31):
         status = 4
     if status == 0 and max_doc_len is not None and longest > max_doc_len:
         status = 5
