@@ -605,7 +605,10 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     // SLOT >= 0: the ring slot of tile i+1 (and with it the p/dz buffer, SLOT and i have opposite
     // parity) is a compile-time constant, so every LDS address is a fixed register plus an
     // immediate; SLOT < 0: taken from i at run time.
-    auto bulk = [&](auto slot_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& set) {
+    // BAND: one of the first steps, whose queries may sit on or above this wave's keys: a key the query must not
+    // see gets r = 1, which makes its p and its dz exactly zero and leaves the stick as it was.
+    auto bulk = [&](auto band_tag, auto slot_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& set) {
+      constexpr bool BAND = decltype(band_tag)::value;
       constexpr int SLOT = decltype(slot_tag)::value;
       constexpr int NCHUNK = 8, PER = 2 * KS / NCHUNK;
       settle(i, set, carry_e, carry_c, dr);   // requested three steps ago
@@ -641,14 +644,22 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       // p / dz fragments this wave's neighbours just staged, and they are the ones the next barrier
       // waits for -- the score waves' own operand reads join one chunk later.
       float r[16], ex[16], p[16];
+      const int qw0 = q_first + i * BQ;
+      const int lim = qw0 + n - k0 - 16 * h + (AC ? 1 : 0);   // (BAND) visible keys of this lane: j < lim
       // chunks 0, 1: r = 1 - beta of the 16 keys
 #pragma unroll
-      for (int j = 0; j < 8; ++j) r[j] = fast_rcp(1.0f + fast_exp2(a.c * xc[j]));
+      for (int j = 0; j < 8; ++j) {
+        r[j] = fast_rcp(1.0f + fast_exp2(a.c * xc[j]));
+        if (BAND && !(j < lim)) r[j] = 1.0f;
+      }
       __builtin_amdgcn_sched_barrier(0);
       pre(0);
       pre(1);
 #pragma unroll
-      for (int j = 8; j < 16; ++j) r[j] = fast_rcp(1.0f + fast_exp2(a.c * xc[j]));
+      for (int j = 8; j < 16; ++j) {
+        r[j] = fast_rcp(1.0f + fast_exp2(a.c * xc[j]));
+        if (BAND && !(j < lim)) r[j] = 1.0f;
+      }
       __builtin_amdgcn_sched_barrier(0);
       // chunk 2: stick left after the newer keys
       pre(2);
@@ -661,8 +672,16 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
 #pragma unroll
       for (int j = 1; j < 16; ++j) p[j] = ex[j] - ex[j - 1];
       el8 pf[2], zf[2];
-      pf[0] = pack8(p);
-      pf[1] = pack8(p + 8);
+      if (BAND && a.fuse && qw0 == k0) {      // (see rem_own)
+        float pd[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) pd[j] = p[j] + (16 * h + j == n ? rem_own : 0.0f);
+        pf[0] = pack8(pd);
+        pf[1] = pack8(pd + 8);
+      } else {
+        pf[0] = pack8(p);
+        pf[1] = pack8(p + 8);
+      }
       post(1);
       // chunk 4: this lane's total of G = sum(p do.v) - drem sum(p), sum(p) = ex[15] - after
       pre(4);
@@ -694,8 +713,19 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       lds_barrier();
     };
     auto later = [&](auto slot_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& set) {
-      if constexpr (PROD && D >= 64) bulk(slot_tag, i, xc, dc, xn, dn, set);   // (its eight chunks need 2 * KS >= 8 chain steps)
+      if constexpr (PROD && D >= 64) bulk(std::false_type{}, slot_tag, i, xc, dc, xn, dn, set);   // (its eight chunks need 2 * KS >= 8 chain steps)
       else step(std::false_type{}, i, xc, dc, xn, dn, set);
+    };
+    auto first = [&](int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& set) {
+      if constexpr (PROD && D >= 64) {
+        // (A block none of whose keys the step's queries may see goes the plain way, which stages zeros without
+        // looking at the carries: the table rows such a step reads are rows of other blocks or rows that nobody
+        // ever wrote, and whatever they hold -- a NaN, say -- must not get anywhere.)
+        if (sub_skip<AC>(k0, q_first + i * BQ)) step(std::true_type{}, i, xc, dc, xn, dn, set);
+        else bulk(std::true_type{}, std::integral_constant<int, -1>{}, i, xc, dc, xn, dn, set);
+      } else {
+        step(std::true_type{}, i, xc, dc, xn, dn, set);
+      }
     };
     // Work queue of a persistent launch, kept by the first score wave ahead of the steps: the draw goes out five
     // steps before the item ends; two steps before the end its answer is taken and the tile descriptor of the
@@ -733,10 +763,10 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       chains(0, xa, da);
       // the first BKV/BQ = 4 steps can touch the diagonal of some wave's block
       queue(0, m & 1);
-      step(std::true_type{}, 0, xa, da, xb, db, r0);
-      if (nsteps > 1) { queue(1, m & 1); step(std::true_type{}, 1, xb, db, xa, da, r1); }
-      if (nsteps > 2) { queue(2, m & 1); step(std::true_type{}, 2, xa, da, xb, db, r2); }
-      if (nsteps > 3) { queue(3, m & 1); step(std::true_type{}, 3, xb, db, xa, da, r0); }
+      first(0, xa, da, xb, db, r0);
+      if (nsteps > 1) { queue(1, m & 1); first(1, xb, db, xa, da, r1); }
+      if (nsteps > 2) { queue(2, m & 1); first(2, xa, da, xb, db, r2); }
+      if (nsteps > 3) { queue(3, m & 1); first(3, xb, db, xa, da, r0); }
       // Whole turns of the ring with static slots (the ring, the two staging buffers, the two
       // accumulator pairs and the three carry sets all repeat with period six: at i = 4 + 6m tile
       // i+1 sits in slot 5 and the carries in set 1), then the remaining steps with run-time slots.
