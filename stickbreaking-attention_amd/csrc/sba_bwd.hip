@@ -466,6 +466,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     int tile_word = -1;
     const bool keeper = persistent && rw == 0;     // (uniform)
     int queue_from = 0x7fffffff;                   // of the current item: the step of the draw (never, for the other waves)
+    int late_tiles = 0;                            // of the current item: tiles this wave copied that may land after its first barrier
     Raw r0, r1, r2;
     // Everything of an item that comes from global memory, requested in one go: the first AHEAD Q / dO
     // tiles, the K and V fragments of this wave's keys and the carries of the first three steps.  For
@@ -506,18 +507,26 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       drem_rs = __builtin_amdgcn_make_buffer_rsrc(a.gtab + tab_rowval, 0, run_bytes, 0x00020000);
       row4 = 4 * (q_first + qr);
       last4 = 4 * (doc_len - 1);
-      if (copier && with_tiles) {
-        const Rows qrows = rows_of(a.q, it), grows = rows_of(a.go, it);
-        Copy qcopy, gcopy;      // (formed here, once per item: a score wave has no register to keep them in)
-        qcopy.init(64 * rw + 32 * h + n, qrows.row_bytes);
-        gcopy.init(64 * rw + 32 * h + n, grows.row_bytes);
+      // In the order of need: the carries of the first steps (small), tiles 0 and 1 and the fragments (all wanted
+      // at the item's first barrier), then the tiles of steps 1 and 2, which only have to arrive one and two steps
+      // later (`late_tiles`, see `guard`).
+      request(0, r0);
+      request(1, r1);
+      request(2, r2);
+      const Rows qrows = rows_of(a.q, it), grows = rows_of(a.go, it);
+      Copy qcopy, gcopy;      // (formed here, once per item: a score wave has no register to keep them in)
+      qcopy.init(64 * rw + 32 * h + n, qrows.row_bytes);
+      gcopy.init(64 * rw + 32 * h + n, grows.row_bytes);
+      auto tiles = [&](int from, int to) {
+        if (!(copier && with_tiles)) return;
 #pragma unroll
-        for (int sft = 0; sft < AHEAD; ++sft)
+        for (int sft = from; sft < to; ++sft)
           if (sft < nsteps) {
             qcopy.issue(qrows, q_first + sft * BQ, Qs + sft * QTILE);
             gcopy.issue(grows, q_first + sft * BQ, Gs + sft * QTILE);
           }
-      }
+      };
+      tiles(0, 2);
       {
         const Rows krows = rows_of(a.k, it), vrows = rows_of(a.v, it);
 #pragma unroll
@@ -526,9 +535,8 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
           vf[ks] = load_frag(vrows, k0 + kperm(n), 32 * ks + 16 * h);
         }
       }
-      request(0, r0);
-      request(1, r1);
-      request(2, r2);
+      tiles(2, AHEAD);
+      late_tiles = with_tiles ? max(min(AHEAD, nsteps) - 2, 0) : 0;
       if (keeper) queue_from = max(nsteps - 5, 0);
     };
     // The row-read offsets of this lane inside a tile (chunk 2*ks + h of row qr).
@@ -548,6 +556,19 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       for (int ks = 0; ks < KS; ++ks) {
         x = mfma32(kf[ks], qfr[ks], x);
         da = mfma32(vf[ks], gfr[ks], da);
+      }
+    };
+    // Ahead of the barrier that ends step 0 (step 1) of an item whose first tiles this wave copied: its part of
+    // tile 2 (tile 3), read behind that barrier, has landed.  What was requested after it -- tile 3 and the
+    // carries of step 3, or the carries of steps 3 and 4 -- may stay in flight (loads return in the order issued).
+    static_assert(AHEAD == 4, "the late tiles are tiles 2 and 3");
+    auto guard = [&](int i) {
+      if (late_tiles == 0 || i > 1) return;
+      if (i == 0) {
+        if (late_tiles == 2) wait_loads<LOADS_PER_TILE + 3>();
+        else wait_loads<3>();
+      } else if (late_tiles == 2) {
+        wait_loads<6>();
       }
     };
     auto stage = [&](int parity, const el8 (&pf)[2], const el8 (&zf)[2]) {
@@ -596,6 +617,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
         grad_dz<PROD>(p, bt, dc, ends, h, carry_c, dr, zf);
       }
       stage(i & 1, pf, zf);
+      if constexpr (DIAG) guard(i);
       lds_barrier();
     };
     // The same step for the product-space carry away from the diagonal, hand-pipelined: the
@@ -710,6 +732,7 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       post(5);
       post(6);
       post(7);
+      if constexpr (BAND) guard(i);
       lds_barrier();
     };
     auto later = [&](auto slot_tag, int i, f32x16& xc, f32x16& dc, f32x16& xn, f32x16& dn, Raw& set) {
@@ -757,7 +780,10 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
     open_item(a, cur, false);     // (a workgroup's first item: the product waves, idle so far, copy its first tiles)
 #pragma unroll 1
     for (int m = 0;; ++m) {
-      wait_loads<9>();                      // all but the carries have arrived: tiles and fragments
+      // the carries, tiles 0 and 1 and the fragments have arrived (not necessarily the late tiles, requested last)
+      if (late_tiles == 2) wait_loads<2 * LOADS_PER_TILE>();
+      else if (late_tiles == 1) wait_loads<LOADS_PER_TILE>();
+      else wait_loads<0>();
       lds_barrier();                        // every score wave's part of tiles 0 .. AHEAD-1 is in slots 0 .. AHEAD-1
       f32x16 xa, da, xb, db;
       chains(0, xa, da);
