@@ -744,8 +744,17 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
         // (A block none of whose keys the step's queries may see goes the plain way, which stages zeros without
         // looking at the carries: the table rows such a step reads are rows of other blocks or rows that nobody
         // ever wrote, and whatever they hold -- a NaN, say -- must not get anywhere.)
-        if (sub_skip<AC>(k0, q_first + i * BQ)) step(std::true_type{}, i, xc, dc, xn, dn, set);
-        else bulk(std::true_type{}, std::integral_constant<int, -1>{}, i, xc, dc, xn, dn, set);
+        if (sub_skip<AC>(k0, q_first + i * BQ)) {
+          settle(i, set, carry_e, carry_c, dr);
+          request(i + 3, set);
+          chains((i + 1) % RING, xn, dn);
+          const el8 zero[2] = {zero8(), zero8()};
+          stage(i & 1, zero, zero);
+          guard(i);
+          lds_barrier();
+        } else {
+          bulk(std::true_type{}, std::integral_constant<int, -1>{}, i, xc, dc, xn, dn, set);
+        }
       } else {
         step(std::true_type{}, i, xc, dc, xn, dn, set);
       }
@@ -800,8 +809,9 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
       int i = BKV / BQ;
       // (the queue's business all falls into an item's last five steps: the turns before them run without it, as one
       // straight-line block)
+      const int spare = persistent ? 5 : 0;
 #pragma unroll 1
-      for (; i + RING + 5 <= nsteps; i += RING) {
+      for (; i + RING + spare <= nsteps; i += RING) {
         later(integral_constant<int, 5>{}, i, xa, da, xb, db, r1);
         later(integral_constant<int, 0>{}, i + 1, xb, db, xa, da, r2);
         later(integral_constant<int, 1>{}, i + 2, xa, da, xb, db, r0);
@@ -809,21 +819,24 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
         later(integral_constant<int, 3>{}, i + 4, xa, da, xb, db, r2);
         later(integral_constant<int, 4>{}, i + 5, xb, db, xa, da, r0);
       }
-#pragma unroll 1
-      for (; i + RING <= nsteps; i += RING) {
-        queue(i, m & 1);     later(integral_constant<int, 5>{}, i, xa, da, xb, db, r1);
-        queue(i + 1, m & 1); later(integral_constant<int, 0>{}, i + 1, xb, db, xa, da, r2);
-        queue(i + 2, m & 1); later(integral_constant<int, 1>{}, i + 2, xa, da, xb, db, r0);
-        queue(i + 3, m & 1); later(integral_constant<int, 2>{}, i + 3, xb, db, xa, da, r1);
-        queue(i + 4, m & 1); later(integral_constant<int, 3>{}, i + 4, xa, da, xb, db, r2);
-        queue(i + 5, m & 1); later(integral_constant<int, 4>{}, i + 5, xb, db, xa, da, r0);
-      }
+      // The item's last steps (five to ten after long runs), with the queue's business between them and ring slots
+      // taken from i at run time: one copy of the step per place in the period of six, walked until the steps run out.
       // (i = 4 + 6m here: accumulator pair a and carry set 1 are next)
-      if (i < nsteps) { queue(i, m & 1); later(integral_constant<int, -1>{}, i, xa, da, xb, db, r1); }
-      if (i + 1 < nsteps) { queue(i + 1, m & 1); later(integral_constant<int, -1>{}, i + 1, xb, db, xa, da, r2); }
-      if (i + 2 < nsteps) { queue(i + 2, m & 1); later(integral_constant<int, -1>{}, i + 2, xa, da, xb, db, r0); }
-      if (i + 3 < nsteps) { queue(i + 3, m & 1); later(integral_constant<int, -1>{}, i + 3, xb, db, xa, da, r1); }
-      if (i + 4 < nsteps) { queue(i + 4, m & 1); later(integral_constant<int, -1>{}, i + 4, xa, da, xb, db, r2); }
+#pragma unroll 1
+      for (;; i += RING) {
+        if (i >= nsteps) break;
+        queue(i, m & 1);     later(integral_constant<int, -1>{}, i, xa, da, xb, db, r1);
+        if (i + 1 >= nsteps) break;
+        queue(i + 1, m & 1); later(integral_constant<int, -1>{}, i + 1, xb, db, xa, da, r2);
+        if (i + 2 >= nsteps) break;
+        queue(i + 2, m & 1); later(integral_constant<int, -1>{}, i + 2, xa, da, xb, db, r0);
+        if (i + 3 >= nsteps) break;
+        queue(i + 3, m & 1); later(integral_constant<int, -1>{}, i + 3, xb, db, xa, da, r1);
+        if (i + 4 >= nsteps) break;
+        queue(i + 4, m & 1); later(integral_constant<int, -1>{}, i + 4, xa, da, xb, db, r2);
+        if (i + 5 >= nsteps) break;
+        queue(i + 5, m & 1); later(integral_constant<int, -1>{}, i + 5, xb, db, xa, da, r0);
+      }
       // This wave is done with the item's tiles and with its K / V fragments: the next item's global
       // reads go out now, while the product waves form the last products and convert and store dk / dv.
       const int next = next_item(m & 1, cur);
