@@ -259,7 +259,7 @@ int backward(const sba_problem* p, bool fixed, const void* schedule, size_t sche
   // fresh workgroup (measured: 960 tiles on 256 compute units, 124 against 118 us).
   const int forced = g_dkdv_workgroups.load();
   a.work = work_words(gtab, table_bytes);
-  a.resident = forced > 0 ? forced : (forced < 0 ? 0 : device_cus());
+  a.resident = forced > 0 ? std::max(8, forced & ~7) : (forced < 0 ? 0 : device_cus());
   a.min_items_each = forced > 0 ? 1 : 8;
   a.max_doc_len = declared_max_doc_len(p, fixed);
   const BwdBounds bb = backward_bounds(p, fixed, sz);

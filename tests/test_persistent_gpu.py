@@ -65,6 +65,26 @@ def test_persistent_launch_matches_one_workgroup_per_tile_bit_for_bit(_lib, d, H
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_random_documents_walked_by_few_workgroups(_lib, seed):
+    """Random splits with many short key tiles (items of one to five steps take every branch of the queue's
+    counted waits and of the late-tile guards), 8 or 24 workgroups for a few hundred items."""
+    import random
+    rng = random.Random(1000 + seed)
+    d = (128, 64, 128, 32)[seed % 4]
+    H = rng.choice((1, 2, 3, 5))
+    lengths = [rng.choice((1, 31, 32, 33, 64, 97, 128, 129, 160, 200, 255, 256, 257, 300, 511, 640, 900)) for _ in range(rng.randint(3, 9))]
+    dev = torch.device("cuda:0")
+    q, k, v, do = (t.to(dev) for t in orc.make_inputs((H, sum(lengths), d), 500 + seed))
+    cu = hp.cu_from_lengths(lengths, device=dev)
+    kw = dict(attend_current=bool(seed & 1))
+    base = _grads_varlen(_lib, -1, q, k, v, do, cu, max(lengths), **kw)
+    for wg in (8, 24):
+        got = _grads_varlen(_lib, wg, q, k, v, do, cu, max(lengths), **kw)
+        for name, a, b in zip(("dq", "dk", "dv"), got, base):
+            assert torch.equal(a, b), f"seed {seed}, lengths {lengths}: {name} differs with {wg} persistent workgroups"
+
+
 def test_persistent_launch_against_the_oracle(_lib):
     dev = torch.device("cuda:0")
     d, H, lengths = 128, 2, [777, 128, 390]
