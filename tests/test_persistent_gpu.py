@@ -85,6 +85,32 @@ def test_random_documents_walked_by_few_workgroups(_lib, seed):
             assert torch.equal(a, b), f"seed {seed}, lengths {lengths}: {name} differs with {wg} persistent workgroups"
 
 
+@pytest.mark.parametrize("d", [128, 64])
+def test_log_space_carry_and_fused_output_with_persistent_workgroups(_lib, monkeypatch, d):
+    """The two other instantiations of the kernel's step: the log2-space carry (no hand-pipelined block at all) and
+    the fused output o + rem * v (rem joins the diagonal of P in the dk/dv pass)."""
+    from stickbreaking_attention import _ops, sb_attn_varlen_fused
+    dev = torch.device("cuda:0")
+    H, lengths = 3, [650, 129, 300, 64]
+    q, k, v, do = (t.to(dev) for t in orc.make_inputs((H, sum(lengths), d), 77 + d))
+    cu = hp.cu_from_lengths(lengths, device=dev)
+    monkeypatch.setattr(_ops, "PRODUCT_SPACE", False)
+    base = _grads_varlen(_lib, -1, q, k, v, do, cu, max(lengths))
+    got = _grads_varlen(_lib, 16, q, k, v, do, cu, max(lengths))
+    for name, a, b in zip(("dq", "dk", "dv"), got, base):
+        assert torch.equal(a, b), f"log space: {name} differs"
+    monkeypatch.setattr(_ops, "PRODUCT_SPACE", True)
+    outs = []
+    for wg in (-1, 16):
+        _lib.sba_set_dkdv_workgroups(wg)
+        qq, kk, vv = (t.detach().clone().requires_grad_() for t in (q, k, v))
+        out = sb_attn_varlen_fused(qq, kk, vv, cu, max(lengths), zero_start=False)
+        outs.append(torch.autograd.grad(out, (qq, kk, vv), do))
+        torch.cuda.synchronize()
+    for name, a, b in zip(("dq", "dk", "dv"), outs[1], outs[0]):
+        assert torch.equal(a, b), f"fused output: {name} differs"
+
+
 def test_persistent_launch_against_the_oracle(_lib):
     dev = torch.device("cuda:0")
     d, H, lengths = 128, 2, [777, 128, 390]
