@@ -39,11 +39,11 @@
 extern "C" {
 #endif
 
-#define SBA_VERSION 211
+#define SBA_VERSION 212
 
 /* error codes (negative returns) */
 #define SBA_E_NULL      (-1)  /* a required pointer is NULL                         */
-#define SBA_E_HEAD_DIM  (-2)  /* head_dim not in {32, 64, 128}                      */
+#define SBA_E_HEAD_DIM  (-2)  /* head_dim not in {32, 64, 128, 256}                 */
 #define SBA_E_DTYPE     (-3)  /* dtype neither SBA_BF16 nor SBA_F16                 */
 #define SBA_E_SHAPE     (-4)  /* negative / inconsistent sizes, or tokens*stride_t
                                  too large for 32-bit byte offsets (>= 2 GiB)       */
@@ -95,7 +95,7 @@ typedef struct sba_view {
 /* Problem description shared by all entry points. */
 typedef struct sba_problem {
   int32_t  dtype;        /* SBA_BF16 or SBA_F16                                          */
-  int32_t  head_dim;     /* 32, 64 or 128                                                */
+  int32_t  head_dim;     /* 32, 64, 128 or 256                                           */
   int32_t  heads;        /* H                                                            */
   int32_t  batch;        /* B for the fixed-length op, 1 for varlen                      */
   int32_t  tokens;       /* T: tokens per batch entry (fixed) / total packed tokens      */

@@ -30,7 +30,7 @@ struct Sizes {
 int check_problem(const sba_problem* p, bool fixed, Sizes* sz) {
   if (p == nullptr) return SBA_E_NULL;
   if (p->dtype != SBA_BF16 && p->dtype != SBA_F16) return SBA_E_DTYPE;
-  if (p->head_dim != 32 && p->head_dim != 64 && p->head_dim != 128) return SBA_E_HEAD_DIM;
+  if (p->head_dim != 32 && p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256) return SBA_E_HEAD_DIM;
   if (p->heads <= 0 || p->tokens < 0 || p->batch <= 0 || p->max_doc_len < 0) return SBA_E_SHAPE;
   if (fixed != ((p->flags & SBA_FIXED_LENGTH) != 0)) return SBA_E_SHAPE;
   if (fixed) {
@@ -315,7 +315,7 @@ const char* sba_error_string(int code) {
   switch (code) {
     case 0: return "ok";
     case SBA_E_NULL: return "a required pointer is NULL";
-    case SBA_E_HEAD_DIM: return "head_dim must be 32, 64 or 128";
+    case SBA_E_HEAD_DIM: return "head_dim must be 32, 64, 128 or 256";
     case SBA_E_DTYPE: return "unsupported element type (SBA_BF16 or SBA_F16)";
     case SBA_E_SHAPE: return "negative or inconsistent sizes";
     case SBA_E_STRIDE: return "pointer or stride breaks 16-byte row alignment";

@@ -103,8 +103,9 @@ __device__ __forceinline__ void grad_dz(const float (&p)[16], const float (&r)[1
 // -------------------------------------------------------------------------------------------
 // dq pass
 // -------------------------------------------------------------------------------------------
+// (head_dim 256: the tiles take 128 KiB, one workgroup per CU, one wave per SIMD with 512 registers)
 template <int D, bool AC, bool PROD>
-__global__ void __launch_bounds__(NT, 2) bwd_dq_kernel(const KArgs a) {
+__global__ void __launch_bounds__(NT, D > 128 ? 1 : 2) bwd_dq_kernel(const KArgs a) {
   constexpr int KS = D / 16, DB = D / 32;
   constexpr int TILE = BN * D;   // elements of one K or V tile (unpadded, swizzled)
   // K (row reads for the scores, transpose reads for dq) and V (row reads) tiles,
@@ -986,14 +987,27 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
 // w, recomputes p and dz of the query blocks at or after it exactly as a score wave does, turns
 // its own 32x32 blocks around through a private piece of LDS and accumulates its own rows of dk
 // and dv.  One barrier (after the Q / dO rows have landed), two workgroups per CU.
+//
+// STREAM: the same four independent waves on EVERY key tile, whatever number of queries follows
+// it: the Q / dO rows then come one query block at a time through two LDS buffers, with one
+// barrier per block.  This is the whole dk/dv pass of head_dim 256, where a wave's K and V
+// fragments (128 registers) and its dk and dv accumulators (256) need the register file of a
+// SIMD to themselves: one workgroup per CU, one wave per SIMD, nothing to split into roles.
 // -------------------------------------------------------------------------------------------
-template <int D, bool AC, bool PROD>
-__global__ void __launch_bounds__(NT, 2) bwd_dkdv_tail_kernel(const KArgs a) {
+template <int D> struct StreamKernel { static constexpr bool value = D > 128; };
+
+template <int D, bool AC, bool PROD, bool STREAM>
+__global__ void __launch_bounds__(NT, D > 128 ? 1 : 2) bwd_dkdv_tail_kernel(const KArgs a) {
   constexpr int KS = D / 16, DB = D / 32;
-  constexpr int QROWS = TAIL_TILES * BKV;            // queries that can follow the tile's first key
+  constexpr int SEG = 32;                             // STREAM: query rows per buffer
+  constexpr int QROWS = STREAM ? 2 * SEG : TAIL_TILES * BKV;   // rows the buffers hold (not STREAM: every query that can follow the tile's first key)
   __shared__ __attribute__((aligned(16))) unsigned short Qs[QROWS * D];   // Q rows from the tile's first key on (swizzled like every tile)
   __shared__ __attribute__((aligned(16))) unsigned short Gs[QROWS * D];   // dO rows
   __shared__ __attribute__((aligned(16))) unsigned short St[NT / 64][2][32 * 32];   // per wave: p and dz of one block, [query][key]
+  // head_dim 256: a wave's dk and dv accumulators fill the 256 accumulation registers and its K fragments 64
+  // of the others; its V fragments wait in LDS instead, in fragment order (wave-private: no barrier involved)
+  constexpr bool V_IN_LDS = D > 128;
+  __shared__ __attribute__((aligned(16))) unsigned short Vf[V_IN_LDS ? NT / 64 : 1][V_IN_LDS ? KS * 64 * 8 : 8];
 
   const int* sched = a.sched;
   const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, table entries needed
@@ -1001,7 +1015,7 @@ __global__ void __launch_bounds__(NT, 2) bwd_dkdv_tail_kernel(const KArgs a) {
   if (hdr.x != 0 || hdr.w > a.tab_stride || hdr2.x > a.max_doc_len) return;
   const int which = blockIdx.x / a.heads;
   const int head = blockIdx.x - which * a.heads;
-  const int slot = hdr2.y + which;
+  const int slot = STREAM ? which : hdr2.y + which;   // STREAM: both groups of the list
   if (slot >= hdr.z) return;
   const Tile t = reinterpret_cast<const Tile*>(sched + a.kv_list_off)[slot];
   const int kt = t.idx;
@@ -1023,25 +1037,34 @@ __global__ void __launch_bounds__(NT, 2) bwd_dkdv_tail_kernel(const KArgs a) {
   const Rows vrows = make_rows(vb, a.v.st, L);
 
   const int q_first = kt * BKV;                      // first query that can see the tile
-  const int nblk = (L - q_first + 31) / 32;          // 1 .. QROWS / 32 query blocks
-  // all of those Q and dO rows at once (rows past the document arrive as zeros)
-  {
-    TileCopy<D, QROWS, NT, false> qcopy, gcopy;
-    qcopy.init(tid, qrows.row_bytes);
-    gcopy.init(tid, grows.row_bytes);
-    qcopy.issue(qrows, q_first, Qs, 32 * nblk);      // (32 or 64 rows per instruction of all waves: whole query blocks)
-    gcopy.issue(grows, q_first, Gs, 32 * nblk);
-  }
+  const int nblk = (L - q_first + 31) / 32;          // query blocks behind the tile's first key (not STREAM: 1 .. QROWS / 32)
+  // all of those Q and dO rows at once, or the first block of them (rows past the document arrive as zeros)
+  TileCopy<D, STREAM ? SEG : QROWS, NT, false> qcopy, gcopy;
+  qcopy.init(tid, qrows.row_bytes);
+  gcopy.init(tid, grows.row_bytes);
+  qcopy.issue(qrows, q_first, Qs, STREAM ? SEG : 32 * nblk);      // (32 or 64 rows per instruction of all waves: whole query blocks)
+  gcopy.issue(grows, q_first, Gs, STREAM ? SEG : 32 * nblk);
   // Wave w of workgroup b takes key block (w + b) mod 4: the block with the most queries behind it
   // is the first one, and two workgroups that share a CU should not both put it on the same SIMD.
   const int kblk = (w + blockIdx.x) & (BKV / 32 - 1);
   const int k0 = q_first + 32 * kblk;                // this wave's keys
   const bool active = k0 < L;
-  el8 kf[KS], vf[KS];                                // MFMA row n holds key k0 + kperm(n)
+  el8 kf[KS], vf[V_IN_LDS ? 1 : KS];                 // MFMA row n holds key k0 + kperm(n)
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     kf[ks] = load_frag(krows, k0 + kperm(n), 32 * ks + 16 * h);
-    vf[ks] = load_frag(vrows, k0 + kperm(n), 32 * ks + 16 * h);
+    if constexpr (!V_IN_LDS) vf[ks] = load_frag(vrows, k0 + kperm(n), 32 * ks + 16 * h);
+  }
+  unsigned short* const Vw = Vf[V_IN_LDS ? w : 0] + 8 * lane;   // this lane's fragment ks at Vw + 512 * ks
+  if constexpr (V_IN_LDS) {
+#pragma unroll
+    for (int c0 = 0; c0 < KS; c0 += 4) {
+      el8 part[4];
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) part[ks] = load_frag(vrows, k0 + kperm(n), 32 * (c0 + ks) + 16 * h);
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) *reinterpret_cast<el8*>(Vw + 512 * (c0 + ks)) = part[ks];
+    }
   }
   // A block that starts past the end of the document is never visible; its table reads are
   // redirected into the document's area and never used.
@@ -1080,21 +1103,19 @@ __global__ void __launch_bounds__(NT, 2) bwd_dkdv_tail_kernel(const KArgs a) {
       yoff[u][j] = swz_off<D>(r, yc >> 3) + (yc & 7);
     }
   }
-  f32x16 acc_v[DB], acc_k[DB];
-#pragma unroll
-  for (int j = 0; j < DB; ++j)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) { acc_v[j][i] = 0.0f; acc_k[j][i] = 0.0f; }
-
-  wait_loads<0>();
-  lds_barrier();              // the only barrier: every wave's part of the Q / dO rows has landed
-  if (!active) return;
+  if constexpr (!STREAM) {
+    wait_loads<0>();
+    lds_barrier();            // the only barrier: every wave's part of the Q / dO rows has landed
+    if (!active) return;
+  }
 
   unsigned short* Pt = St[w][0];
   unsigned short* Zt = St[w][1];
-  // query blocks at or after the key block (those before it see none of these keys)
-#pragma unroll 1
-  for (int qblk = kblk; qblk < nblk; ++qblk) {
+  // Query block qblk, whose Q / dO rows begin at buffer row lrow0.  WHAT: 0 = p alone and its
+  // products into `acc` (dv), 1 = dz alone and its products into `acc` (dk), 2 = both, dk into `acc2`.
+  auto block = [&](auto what_tag, f32x16 (&acc)[DB], f32x16 (&acc2)[DB], const int qblk, const int lrow0) {
+    constexpr int WHAT = decltype(what_tag)::value;
+    constexpr bool DV = WHAT != 1, DK = WHAT != 0;
     request(qblk + 1, nxt);                           // (clamped; unused past the last block)
     const int qw0 = q_first + 32 * qblk;
     const int qrow = qw0 + n;
@@ -1106,62 +1127,126 @@ __global__ void __launch_bounds__(NT, 2) bwd_dkdv_tail_kernel(const KArgs a) {
 #pragma unroll
     for (int j = 0; j < 16; ++j) { x[j] = 0.0f; da[j] = 0.0f; }
     {
-      const unsigned short* Qt = Qs + 32 * qblk * D;
-      const unsigned short* Gt = Gs + 32 * qblk * D;
-      el8 qfr[KS], gfr[KS];
+      const unsigned short* Qt = Qs + lrow0 * D;
+      const unsigned short* Gt = Gs + lrow0 * D;
+      // (head_dim 256: four contraction steps at a time, so that the operand fragments of a whole
+      // chain are never in registers at once)
+      constexpr int CH = D > 128 ? 4 : KS;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) { qfr[ks] = lds_row8(Qt + roff[ks]); gfr[ks] = lds_row8(Gt + roff[ks]); }
+      for (int c0 = 0; c0 < KS; c0 += CH) {
+        el8 qfr[CH], gfr[CH];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        x = mfma32(kf[ks], qfr[ks], x);
-        da = mfma32(vf[ks], gfr[ks], da);
+        for (int ks = 0; ks < CH; ++ks) {
+          qfr[ks] = lds_row8(Qt + roff[c0 + ks]);
+          if constexpr (DK) gfr[ks] = lds_row8(Gt + roff[c0 + ks]);
+        }
+#pragma unroll
+        for (int ks = 0; ks < CH; ++ks) {
+          x = mfma32(kf[c0 + ks], qfr[ks], x);
+          if constexpr (DK) {
+            if constexpr (V_IN_LDS) da = mfma32(lds_row8(Vw + 512 * (c0 + ks)), gfr[ks], da);
+            else da = mfma32(vf[c0 + ks], gfr[ks], da);
+          }
+        }
+        if constexpr (D > 128) __builtin_amdgcn_sched_barrier(0);
       }
     }
     el8 pf[2], zf[2];
     {
       float p[16], bt[16], ends[2] = {0.0f, 0.0f};
       grad_weights<AC, PROD>(x, a.c, k0, qw0, qrow, h, carry_e, p, bt, ends);
-      if (a.fuse && qblk == kblk) {
-        float pd[16];
+      if constexpr (DV) {
+        if (a.fuse && qblk == kblk) {
+          float pd[16];
 #pragma unroll
-        for (int j = 0; j < 16; ++j) pd[j] = p[j] + (16 * h + j == n ? rem_own : 0.0f);
-        pf[0] = pack8(pd);
-        pf[1] = pack8(pd + 8);
-      } else {
-        pf[0] = pack8(p);
-        pf[1] = pack8(p + 8);
+          for (int j = 0; j < 16; ++j) pd[j] = p[j] + (16 * h + j == n ? rem_own : 0.0f);
+          pf[0] = pack8(pd);
+          pf[1] = pack8(pd + 8);
+        } else {
+          pf[0] = pack8(p);
+          pf[1] = pack8(p + 8);
+        }
       }
-      grad_dz<PROD>(p, bt, da, ends, h, carry_c, dr, zf);
+      if constexpr (DK) grad_dz<PROD>(p, bt, da, ends, h, carry_c, dr, zf);
     }
     // turn the block around: [query][key] rows in, key-major MFMA operands out
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
-      *reinterpret_cast<el8*>(Pt + blk_off(n, 2 * h + tt)) = pf[tt];
-      *reinterpret_cast<el8*>(Zt + blk_off(n, 2 * h + tt)) = zf[tt];
+      if constexpr (DV) *reinterpret_cast<el8*>(Pt + blk_off(n, 2 * h + tt)) = pf[tt];
+      if constexpr (DK) *reinterpret_cast<el8*>(Zt + blk_off(n, 2 * h + tt)) = zf[tt];
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own writes have landed
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      const el8 ap = lds_tr8(Pt + xoff[0] + 16 * ks * 32, Pt + xoff[1] + 16 * ks * 32);
-      const el8 az = lds_tr8(Zt + xoff[0] + 16 * ks * 32, Zt + xoff[1] + 16 * ks * 32);
-      const unsigned short* Gr = Gs + (32 * qblk + 16 * ks) * D;
-      const unsigned short* Qr = Qs + (32 * qblk + 16 * ks) * D;
+      el8 ap, az;
+      if constexpr (DV) ap = lds_tr8(Pt + xoff[0] + 16 * ks * 32, Pt + xoff[1] + 16 * ks * 32);
+      if constexpr (DK) az = lds_tr8(Zt + xoff[0] + 16 * ks * 32, Zt + xoff[1] + 16 * ks * 32);
+      const unsigned short* Gr = Gs + (lrow0 + 16 * ks) * D;
+      const unsigned short* Qr = Qs + (lrow0 + 16 * ks) * D;
 #pragma unroll
       for (int j = 0; j < DB; ++j) {
-        acc_v[j] = mfma32(ap, lds_tr8(Gr + yoff[0][j], Gr + yoff[1][j]), acc_v[j]);
-        acc_k[j] = mfma32(az, lds_tr8(Qr + yoff[0][j], Qr + yoff[1][j]), acc_k[j]);
+        if constexpr (DV) acc[j] = mfma32(ap, lds_tr8(Gr + yoff[0][j], Gr + yoff[1][j]), acc[j]);
+        if constexpr (WHAT == 1) acc[j] = mfma32(az, lds_tr8(Qr + yoff[0][j], Qr + yoff[1][j]), acc[j]);
+        if constexpr (WHAT == 2) acc2[j] = mfma32(az, lds_tr8(Qr + yoff[0][j], Qr + yoff[1][j]), acc2[j]);
+        if constexpr (D > 128) { if (j % 4 == 3) __builtin_amdgcn_sched_barrier(0); }
       }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the reads are done before the next block overwrites the piece
     cur = nxt;
-  }
-  // the private piece becomes the output scratch (32 x D elements: at most its size)
-  static_assert(2 * 32 * 32 >= 32 * D, "the staging piece of a wave doubles as its output scratch");
+  };
+  auto clear = [&](f32x16 (&acc)[DB]) {
+#pragma unroll
+    for (int j = 0; j < DB; ++j)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[j][i] = 0.0f;
+  };
   elem_t* dvb = reinterpret_cast<elem_t*>(a.dv.ptr) + t.batch * a.dv.sb + head * a.dv.sh + tok0 * a.dv.st;
   elem_t* dkb = reinterpret_cast<elem_t*>(a.dk.ptr) + t.batch * a.dk.sb + head * a.dk.sh + tok0 * a.dk.st;
-  store_block32<D>(Pt, acc_v, 1.0f, dvb, a.dv.st, k0, L, lane);
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  store_block32<D>(Pt, acc_k, a.inv_temp, dkb, a.dk.st, k0, L, lane);
+  if constexpr (!STREAM) {
+    f32x16 acc_v[DB], acc_k[DB];
+    clear(acc_v);
+    clear(acc_k);
+    // query blocks at or after the key block (those before it see none of these keys)
+#pragma unroll 1
+    for (int qblk = kblk; qblk < nblk; ++qblk) block(std::integral_constant<int, 2>{}, acc_v, acc_k, qblk, 32 * qblk);
+    // the private piece becomes the output scratch (at most its size)
+    static_assert(STREAM || 2 * 32 * 32 >= 32 * D, "the staging piece of a wave doubles as its output scratch");
+    store_block32<D>(Pt, acc_v, 1.0f, dvb, a.dv.st, k0, L, lane);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    store_block32<D>(Pt, acc_k, a.inv_temp, dkb, a.dk.st, k0, L, lane);
+  } else {
+    // Two passes over the queries, dv first and dk second: one output's accumulators (128 registers at
+    // head_dim 256) beside the chains' own, instead of both.  The scores are formed in each pass.
+    // Query block s sits in buffer s & 1.  At its top every wave is done with block s - 1, whose buffer
+    // takes the rows of block s + 1 while this one is worked on.
+    static_assert(!STREAM || (QROWS == 64 && NT / 64 == 4), "a quarter of the two buffers per wave for its output");
+    unsigned short* const scratch = (w & 2 ? Gs : Qs) + (w & 1) * 32 * D;
+    auto pass = [&](auto what_tag) {
+      f32x16 acc[DB];
+      clear(acc);
+#pragma unroll 1
+      for (int qblk = 0; qblk < nblk; ++qblk) {
+        wait_loads<0>();
+        lds_barrier();
+        if (qblk + 1 < nblk) {
+          qcopy.issue(qrows, q_first + (qblk + 1) * SEG, Qs + ((qblk + 1) & 1) * SEG * D);
+          gcopy.issue(grows, q_first + (qblk + 1) * SEG, Gs + ((qblk + 1) & 1) * SEG * D);
+        }
+        if (active && qblk >= kblk) block(what_tag, acc, acc, qblk, (qblk & 1) * SEG);
+      }
+      lds_barrier();            // every wave is done with the buffers: they become the output staging
+      if (active) {
+        if constexpr (decltype(what_tag)::value == 0) store_block32<D>(scratch, acc, 1.0f, dvb, a.dv.st, k0, L, lane);
+        else store_block32<D>(scratch, acc, a.inv_temp, dkb, a.dk.st, k0, L, lane);
+      }
+    };
+    pass(std::integral_constant<int, 0>{});
+    lds_barrier();              // and buffers again: the first block's rows once more
+    qcopy.issue(qrows, q_first, Qs, SEG);
+    gcopy.issue(grows, q_first, Gs, SEG);
+    request(kblk, cur);
+    pass(std::integral_constant<int, 1>{});
+  }
 }
 
 // Explicit instantiations: every (head_dim, attend_current, carry space) variant the launchers use.
@@ -1177,14 +1262,22 @@ template __global__ void bwd_dq_kernel<128, false, false>(const KArgs);
 template __global__ void bwd_dq_kernel<128, false, true>(const KArgs);
 template __global__ void bwd_dq_kernel<128, true, false>(const KArgs);
 template __global__ void bwd_dq_kernel<128, true, true>(const KArgs);
-template __global__ void bwd_dkdv_tail_kernel<32, false, false>(const KArgs);
-template __global__ void bwd_dkdv_tail_kernel<32, false, true>(const KArgs);
-template __global__ void bwd_dkdv_tail_kernel<32, true, false>(const KArgs);
-template __global__ void bwd_dkdv_tail_kernel<32, true, true>(const KArgs);
-template __global__ void bwd_dkdv_tail_kernel<64, false, false>(const KArgs);
-template __global__ void bwd_dkdv_tail_kernel<64, false, true>(const KArgs);
-template __global__ void bwd_dkdv_tail_kernel<64, true, false>(const KArgs);
-template __global__ void bwd_dkdv_tail_kernel<64, true, true>(const KArgs);
+template __global__ void bwd_dq_kernel<256, false, false>(const KArgs);
+template __global__ void bwd_dq_kernel<256, false, true>(const KArgs);
+template __global__ void bwd_dq_kernel<256, true, false>(const KArgs);
+template __global__ void bwd_dq_kernel<256, true, true>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<256, false, false, true>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<256, false, true, true>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<256, true, false, true>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<256, true, true, true>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<32, false, false, false>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<32, false, true, false>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<32, true, false, false>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<32, true, true, false>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<64, false, false, false>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<64, false, true, false>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<64, true, false, false>(const KArgs);
+template __global__ void bwd_dkdv_tail_kernel<64, true, true, false>(const KArgs);
 template __global__ void bwd_dkdv_kernel<32, false, false>(const KArgs);
 template __global__ void bwd_dkdv_kernel<32, false, true>(const KArgs);
 template __global__ void bwd_dkdv_kernel<32, true, false>(const KArgs);
@@ -1212,39 +1305,49 @@ static hipError_t launch_dq_d(const KArgs& a, bool ac, bool prod, int n_q_max, h
 }
 
 // n_long_max / n_last_max: upper bounds on the key tiles of the first / second group of the list.
+template <int D, bool STREAM>
+static void launch_dkdv_four_waves(const KArgs& a, bool ac, bool prod, unsigned tiles, hipStream_t s) {
+  const dim3 grid(tiles * (unsigned)a.heads), block(NT);
+  if (ac) {
+    if (prod) hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, true, true, STREAM>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, true, false, STREAM>), grid, block, 0, s, a);
+  } else {
+    if (prod) hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, false, true, STREAM>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, false, false, STREAM>), grid, block, 0, s, a);
+  }
+}
+
+// n_long_max / n_last_max: upper bounds on the key tiles of the first / second group of the list.
 template <int D>
 static hipError_t launch_dkdv_d(const KArgs& a_in, bool ac, bool prod, int n_long_max, int n_last_max, hipStream_t s) {
   static_assert(TailKernel<D>::value == (D <= 64), "has_dkdv_tail_kernel() states the same rule for the host");
   KArgs a = a_in;
   const DkdvGrid g = dkdv_grid(TailKernel<D>::value, n_long_max, n_last_max, a.n_kv_alloc);
   const unsigned n_main = (unsigned)g.main_tiles;
-  if (n_main > 0) {
-    a.n_items = (int)(n_main * (unsigned)a.heads);
-    const dim3 grid(launch_grid(a, a.n_items)), block(NT2);
-    if (ac) {
-      if (prod) hipLaunchKernelGGL((bwd_dkdv_kernel<D, true, true>), grid, block, 0, s, a);
-      else hipLaunchKernelGGL((bwd_dkdv_kernel<D, true, false>), grid, block, 0, s, a);
-    } else {
-      if (prod) hipLaunchKernelGGL((bwd_dkdv_kernel<D, false, true>), grid, block, 0, s, a);
-      else hipLaunchKernelGGL((bwd_dkdv_kernel<D, false, false>), grid, block, 0, s, a);
-    }
-  }
-  if constexpr (TailKernel<D>::value) {
-    if (g.tail_tiles > 0) {
-      const dim3 grid((unsigned)g.tail_tiles * (unsigned)a.heads), block(NT);
+  if constexpr (StreamKernel<D>::value) {
+    // every key tile of both groups to the four independent waves, queries streamed
+    if (n_main > 0) launch_dkdv_four_waves<D, true>(a, ac, prod, n_main, s);
+  } else {
+    if (n_main > 0) {
+      a.n_items = (int)(n_main * (unsigned)a.heads);
+      const dim3 grid(launch_grid(a, a.n_items)), block(NT2);
       if (ac) {
-        if (prod) hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, true, true>), grid, block, 0, s, a);
-        else hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, true, false>), grid, block, 0, s, a);
+        if (prod) hipLaunchKernelGGL((bwd_dkdv_kernel<D, true, true>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((bwd_dkdv_kernel<D, true, false>), grid, block, 0, s, a);
       } else {
-        if (prod) hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, false, true>), grid, block, 0, s, a);
-        else hipLaunchKernelGGL((bwd_dkdv_tail_kernel<D, false, false>), grid, block, 0, s, a);
+        if (prod) hipLaunchKernelGGL((bwd_dkdv_kernel<D, false, true>), grid, block, 0, s, a);
+        else hipLaunchKernelGGL((bwd_dkdv_kernel<D, false, false>), grid, block, 0, s, a);
       }
+    }
+    if constexpr (TailKernel<D>::value) {
+      if (g.tail_tiles > 0) launch_dkdv_four_waves<D, false>(a, ac, prod, (unsigned)g.tail_tiles, s);
     }
   }
   return hipGetLastError();
 }
 
 hipError_t launch_bwd_dq(const KArgs& a, int head_dim, bool ac, bool prod, int n_q_max, hipStream_t s) {
+  if (head_dim == 256) return launch_dq_d<256>(a, ac, prod, n_q_max, s);
   if (head_dim == 128) return launch_dq_d<128>(a, ac, prod, n_q_max, s);
   if (head_dim == 64) return launch_dq_d<64>(a, ac, prod, n_q_max, s);
   return launch_dq_d<32>(a, ac, prod, n_q_max, s);
@@ -1252,6 +1355,7 @@ hipError_t launch_bwd_dq(const KArgs& a, int head_dim, bool ac, bool prod, int n
 
 hipError_t launch_bwd_dkdv(const KArgs& a, int head_dim, bool ac, bool prod, int n_long_max, int n_last_max,
                            hipStream_t s) {
+  if (head_dim == 256) return launch_dkdv_d<256>(a, ac, prod, n_long_max, n_last_max, s);
   if (head_dim == 128) return launch_dkdv_d<128>(a, ac, prod, n_long_max, n_last_max, s);
   if (head_dim == 64) return launch_dkdv_d<64>(a, ac, prod, n_long_max, n_last_max, s);
   return launch_dkdv_d<32>(a, ac, prod, n_long_max, n_last_max, s);

@@ -532,7 +532,8 @@ __device__ __forceinline__ el8 load_frag(const Rows& r, int row, int col_bytes) 
 // one chunk each) and transpose reads (4 consecutive rows, 64 contiguous bytes each).
 template <int D>
 __device__ __forceinline__ int swz(int row) {
-  if constexpr (D == 128) return ((row & 3) << 2) | ((row >> 2) & 3);
+  // (512-byte rows span the banks twice: the chunk's low four bits decide its banks, as with 256-byte rows)
+  if constexpr (D >= 128) return ((row & 3) << 2) | ((row >> 2) & 3);
   else if constexpr (D == 64) { const int x = (row >> 1) & 7; return ((x & 1) << 2) | (x >> 1); }
   else return (row >> 2) & 3;   // 64-byte rows: four rows fill the banks, the next four take the next rotation
 }
@@ -578,13 +579,20 @@ struct TileCopy {
   static constexpr int NCH = ROWS * C8 / THREADS;
   static constexpr int RPI = 64 / C8;                 // rows one wave instruction covers
   static constexpr int STEP = (THREADS / 64) * RPI;   // rows one instruction of every wave covers
+  // 512-byte rows with four loading waves: STEP is 8, the swizzle of a row repeats every 16 rows, so the
+  // instructions with odd j need a second per-lane offset (the swizzle's bit 1 flipped)
+  static constexpr bool TWO_PHASE = STEP == 8;
   static_assert(ROWS * C8 % THREADS == 0, "tile must split evenly over the loading threads");
-  static_assert(STEP % 16 == 0 && (NCH == 1 || STEP == 16 || STEP % 32 == 0), "row step must be invisible to the swizzle");
-  int voff;    // byte offset of this lane's chunk in instruction 0, relative to the tile's first row
+  static_assert(TWO_PHASE ? (D == 256 && RPI == 2)
+                          : (STEP % 16 == 0 && (NCH == 1 || STEP == 16 || STEP % 32 == 0)), "row step must be invisible to the swizzle");
+  int voff;       // byte offset of this lane's chunk in instruction 0, relative to the tile's first row
+  int voff_odd;   // TWO_PHASE: the same for instructions with odd j (relative to that instruction's first row)
   int wave;
 
   // source row offset of instruction j relative to instruction 0
   static constexpr int row_delta(int j) {
+    // STEP == 8: bits 3 and 4 of the tile row become bits 2 and 3 of the permuted key (see kperm)
+    if (TWO_PHASE) return KEYS ? 32 * (j >> 2) + 4 * (j & 3) : j * STEP;
     if (!KEYS || STEP % 32 == 0) return j * STEP;
     // STEP == 16: bit 4 of the tile row becomes bit 3 of the permuted key (see kperm)
     return 32 * (j >> 1) + 8 * (j & 1);
@@ -598,6 +606,7 @@ struct TileCopy {
     const int logical = phys ^ swz<D>(m);
     const int src = KEYS ? ((m & ~31) | kperm(m & 31)) : m;
     voff = src * (int)row_bytes + logical * 16;
+    voff_odd = src * (int)row_bytes + (phys ^ swz<D>(m + 8)) * 16;
   }
 
   // `rows_needed` (uniform): instructions whose rows all lie at or beyond it are skipped; the tile
@@ -610,9 +619,9 @@ struct TileCopy {
 #ifdef SBA_BUILTIN_DMA
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
           r.rsrc, (__attribute__((address_space(3))) void*)(lds_tile + (j * STEP + wave * RPI) * D), 16,
-          voff, soff, 0, 0);
+          TWO_PHASE && (j & 1) ? voff_odd : voff, soff, 0, 0);
 #else
-      async_copy16(r.rsrc, lds_tile + (j * STEP + wave * RPI) * D, voff, soff);
+      async_copy16(r.rsrc, lds_tile + (j * STEP + wave * RPI) * D, TWO_PHASE && (j & 1) ? voff_odd : voff, soff);
 #endif
     }
   }

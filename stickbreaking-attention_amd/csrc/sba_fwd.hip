@@ -16,15 +16,17 @@ inline namespace SBA_ELEM_NS {
 // (sb_varlen_fwd.py:195-202).  MODE 2 (TAB): write the carry table and nothing else -- no V tiles,
 // no P.V products, no o, no rem -- for a backward whose forward kept no table.  Separate
 // instantiations, so the production kernel (MODE 0) carries none of it.
+// head_dim 256: the ring takes 96 KiB, so one workgroup per CU and one wave per SIMD, with the whole register
+// file (512 registers per lane) for its 64 registers of Q fragments and 128 of accumulators.
 template <int D, bool AC, bool PROD, int MODE>
-__global__ void __launch_bounds__(NT, 3) fwd_kernel(const KArgs a) {
+__global__ void __launch_bounds__(NT, D > 128 ? 1 : 3) fwd_kernel(const KArgs a) {
   constexpr bool WOUT = MODE == 1, TAB = MODE == 2;
   constexpr int KS = D / 16;     // contraction steps of K.Q^T
   constexpr int DB = D / 32;     // 32-wide output column blocks of P.V
   constexpr int BF = 32;         // keys per staged tile: one MFMA sub-block
   constexpr int TILE = BF * D;   // elements of one K or V tile (unpadded, swizzled)
   // K and V tiles of 32 keys in a three-slot ring filled by asynchronous global -> LDS copies:
-  // 48 KiB per workgroup, so three workgroups share a CU.
+  // 48 KiB per workgroup at head_dim 128, so three workgroups share a CU.
   __shared__ __attribute__((aligned(16))) unsigned short smem[6 * TILE];
   unsigned short* const Ks = smem;              // three K tiles
   unsigned short* const Vs = smem + 3 * TILE;   // three V tiles
@@ -254,6 +256,18 @@ template __global__ void fwd_kernel<128, false, false, 2>(const KArgs);
 template __global__ void fwd_kernel<128, false, true, 2>(const KArgs);
 template __global__ void fwd_kernel<128, true, false, 2>(const KArgs);
 template __global__ void fwd_kernel<128, true, true, 2>(const KArgs);
+template __global__ void fwd_kernel<256, false, false, 0>(const KArgs);
+template __global__ void fwd_kernel<256, false, false, 1>(const KArgs);
+template __global__ void fwd_kernel<256, false, true, 0>(const KArgs);
+template __global__ void fwd_kernel<256, false, true, 1>(const KArgs);
+template __global__ void fwd_kernel<256, true, false, 0>(const KArgs);
+template __global__ void fwd_kernel<256, true, false, 1>(const KArgs);
+template __global__ void fwd_kernel<256, true, true, 0>(const KArgs);
+template __global__ void fwd_kernel<256, true, true, 1>(const KArgs);
+template __global__ void fwd_kernel<256, false, false, 2>(const KArgs);
+template __global__ void fwd_kernel<256, false, true, 2>(const KArgs);
+template __global__ void fwd_kernel<256, true, false, 2>(const KArgs);
+template __global__ void fwd_kernel<256, true, true, 2>(const KArgs);
 
 template <int D, int MODE>
 static hipError_t launch_fwd_d(const KArgs& a, bool ac, bool prod, int n_q_max, hipStream_t s) {
@@ -271,15 +285,18 @@ static hipError_t launch_fwd_d(const KArgs& a, bool ac, bool prod, int n_q_max, 
 // mode: 0 = o and rem (and the table when one is given), 1 = the attention weights as well, 2 = the table alone
 hipError_t launch_fwd(const KArgs& a, int head_dim, bool ac, bool prod, int mode, int n_q_max, hipStream_t s) {
   if (mode == 1) {
+    if (head_dim == 256) return launch_fwd_d<256, 1>(a, ac, prod, n_q_max, s);
     if (head_dim == 128) return launch_fwd_d<128, 1>(a, ac, prod, n_q_max, s);
     if (head_dim == 64) return launch_fwd_d<64, 1>(a, ac, prod, n_q_max, s);
     return launch_fwd_d<32, 1>(a, ac, prod, n_q_max, s);
   }
   if (mode == 2) {
+    if (head_dim == 256) return launch_fwd_d<256, 2>(a, ac, prod, n_q_max, s);
     if (head_dim == 128) return launch_fwd_d<128, 2>(a, ac, prod, n_q_max, s);
     if (head_dim == 64) return launch_fwd_d<64, 2>(a, ac, prod, n_q_max, s);
     return launch_fwd_d<32, 2>(a, ac, prod, n_q_max, s);
   }
+  if (head_dim == 256) return launch_fwd_d<256, 0>(a, ac, prod, n_q_max, s);
   if (head_dim == 128) return launch_fwd_d<128, 0>(a, ac, prod, n_q_max, s);
   if (head_dim == 64) return launch_fwd_d<64, 0>(a, ac, prod, n_q_max, s);
   return launch_fwd_d<32, 0>(a, ac, prod, n_q_max, s);

@@ -49,7 +49,7 @@ SYNC_FREE = os.environ.get("SBA_SYNC_FREE", "0") == "1"
 # rebuilt table is one scratch buffer shared by all layers.
 RECOMPUTE_TABLE = os.environ.get("SBA_RECOMPUTE_TABLE", "0") == "1"
 
-SUPPORTED_HEAD_DIMS = (32, 64, 128)
+SUPPORTED_HEAD_DIMS = (32, 64, 128, 256)
 
 # Tile sizes the library's workspace formulas are built on (query tile, dk/dv key tile, table block).
 _BM, _BKV, _BT, _SCHED_HDR, _TILE_WORDS = 128, 128, 32, 16, 8

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for s in syms:
         assert hasattr(lib, s), f"{s} declared in include/sba.h but not exported"
     assert sorted(nat.EXPORTS) == syms
-    assert lib.sba_version() == 211
+    assert lib.sba_version() == 212
 
 
 def problem(**kw):
@@ -121,7 +121,7 @@ def test_table_only_forward_checks_its_arguments():
 
 
 @pytest.mark.parametrize("kw,code", [
-    (dict(head_dim=50), -2), (dict(dtype=7), -3), (dict(dtype=2, head_dim=50), -2), (dict(heads=0), -4), (dict(batch=2), -4),
+    (dict(head_dim=50), -2), (dict(head_dim=512), -2), (dict(dtype=7), -3), (dict(dtype=2, head_dim=50), -2), (dict(heads=0), -4), (dict(batch=2), -4),
     (dict(cu_seqlens=None), -1),
 ])
 def test_bad_problems_are_rejected_on_the_host(kw, code):
@@ -301,7 +301,7 @@ def test_every_launch_stays_inside_the_schedule_workspace():
         mdl = rng.choice([0, 1, rng.randint(0, max(tokens, 1)), tokens, tokens + 7])
         cases.append((tokens, n_docs, mdl))
     for tokens, n_docs, mdl in cases:
-        for d in (32, 64, 128):
+        for d in (32, 64, 128, 256):
             g = _geometry(tokens=tokens, n_docs=n_docs, max_doc_len=mdl, head_dim=d, heads=3)
             _check_geometry(g, n_docs)
             # what an earlier version launched at head_dim 128 (both bounds added, no clamp) does NOT stay inside:
@@ -310,7 +310,7 @@ def test_every_launch_stays_inside_the_schedule_workspace():
     assert g.long_tiles_bound + g.tail_tiles_bound > g.key_list_tiles >= g.dkdv_main_tiles
     # fixed length: batch documents of `tokens` tokens each
     for batch, tokens in [(1, 1), (4, 2048), (3, 500), (2, 16384), (7, 129)]:
-        for d in (32, 64, 128):
+        for d in (32, 64, 128, 256):
             g = _geometry(batch=batch, tokens=tokens, n_docs=0, max_doc_len=tokens, head_dim=d, heads=2,
                           flags=nat.FLAG_FIXED_LENGTH, cu_seqlens=None)
             _check_geometry(g, batch)
@@ -330,7 +330,7 @@ def test_launch_bounds_cover_every_split_into_documents():
         else: lengths = [int(2 ** rng.uniform(0, 13)) for _ in range(n_docs)]
         tokens = sum(lengths) + rng.choice([0, 0, 5, 300])      # rows behind the last document are allowed
         mdl = max(lengths)
-        for d in (64, 128):
+        for d in (64, 128, 256):
             g = _geometry(tokens=tokens, n_docs=n_docs, max_doc_len=mdl, head_dim=d, heads=1)
             assert _tiles(lengths, 128) <= g.fwd_tiles
             n_kv = _tiles(lengths, 128)
@@ -338,7 +338,7 @@ def test_launch_bounds_cover_every_split_into_documents():
             n_tail = sum(_tail_tiles(n) for n in lengths if n > 0)
             n_long = n_kv - n_tail
             assert n_long <= g.long_tiles_bound and n_tail <= g.tail_tiles_bound
-            if d == 128:
+            if d >= 128:
                 assert n_kv <= g.dkdv_main_tiles           # one kernel takes both groups
             else:
                 assert n_long <= g.dkdv_main_tiles and n_tail <= g.dkdv_tail_tiles

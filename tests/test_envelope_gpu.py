@@ -36,7 +36,7 @@ def _run(q, k, v, do, lengths, ac=False):
 
 @pytest.mark.parametrize("product_space", [False, True])
 @pytest.mark.parametrize("qk_scale", [3.0, 8.0])
-@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("d", [64, 128, 256])
 def test_large_logits(product_space, qk_scale, d, monkeypatch):
     """q and k scaled so that the logits reach +-35 (x3) or +-250 (x8): sigmoid saturates, 2^z
     overflows fp32 (product space: r = 0; log2 space: logit clamped at 126), the forward's clamp
@@ -81,7 +81,7 @@ def test_fp32_inputs_are_rounded_to_bf16_and_say_so():
         assert_close(name + " (fp32 inputs)", gt, r)
 
 
-@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
 def test_float16_runs_on_the_float16_kernels(d):
     """float16 q, k, v, grad_o are multiplied as float16 (11 significant bits instead of bfloat16's 8;
     upstream's tl.dot does the same, sb_varlen_fwd.py:42): the operands P and dZ and the outputs are

@@ -52,7 +52,7 @@ def run_fused_varlen(q, k, v, dout, lengths, ac=False, prepare=lambda t: t.to(DE
 
 @pytest.mark.parametrize("lengths", [[1], [3, 1, 1, 2], [63, 64, 65, 127, 128, 129, 1, 31, 33], [257, 640]])
 @pytest.mark.parametrize("ac", [False, True])
-@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
 def test_fused_varlen_ragged_documents(lengths, ac, d):
     T = sum(lengths)
     q, k, v, dout = orc.make_inputs((3, T, d), 11 + T + d, dist="upstream")
@@ -68,7 +68,7 @@ def test_fused_varlen_long_documents_normal_inputs(product_space, monkeypatch):
     check(run_fused_varlen(q, k, v, dout, lengths), fused_reference(q, k, v, dout, lengths))
 
 
-@pytest.mark.parametrize("B,H,T,d,ac", [(2, 3, 200, 64, False), (1, 2, 384, 128, True), (2, 2, 300, 32, True)])
+@pytest.mark.parametrize("B,H,T,d,ac", [(2, 3, 200, 64, False), (1, 2, 384, 128, True), (2, 2, 300, 32, True), (1, 2, 450, 256, False)])
 def test_fused_fixed_length(B, H, T, d, ac):
     from stickbreaking_attention import sb_attn_fused
     q, k, v, dout = orc.make_inputs((B, H, T, d), 3 + T, dist="upstream")

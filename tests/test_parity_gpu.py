@@ -92,7 +92,7 @@ def test_log_space_carry_on_long_documents(ac, monkeypatch):
 
 @pytest.mark.parametrize("lengths", [[1], [2], [3, 1, 1, 2], [63, 64, 65, 127, 128, 129, 1, 31, 33], [257, 640]])
 @pytest.mark.parametrize("ac", [False, True])
-@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
 def test_ragged_documents(lengths, ac, d):
     T = sum(lengths)
     q, k, v, do = orc.make_inputs((3, T, d), 7 + T + d, dist="upstream")
@@ -201,7 +201,7 @@ def test_empty_documents_and_tail_tokens():
 
 
 @pytest.mark.parametrize("ac", [False, True])
-@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
 def test_key_tile_group_boundaries(d, ac, monkeypatch):
     """Document lengths on both sides of every boundary of the dk/dv pass's tile grouping (all key
     tiles of a document of up to 256 tokens and the last tile of a longer one go to the four-wave
@@ -244,7 +244,8 @@ def test_upstream_varlen_grid(H, L, ac):
 
 
 @pytest.mark.parametrize("ac", [False, True])
-@pytest.mark.parametrize("B,H,T,d", [(2, 3, 500, 64), (1, 7, 256, 64), (2, 2, 1024, 128), (2, 3, 700, 32), (1, 2, 2048, 32)])
+@pytest.mark.parametrize("B,H,T,d", [(2, 3, 500, 64), (1, 7, 256, 64), (2, 2, 1024, 128), (2, 3, 700, 32), (1, 2, 2048, 32),
+                                     (2, 2, 700, 256)])
 def test_fixed_length(B, H, T, d, ac):
     from stickbreaking_attention import sb_attn
     q, k, v, do = orc.make_inputs((B, H, T, d), 5 + T, dist="upstream")
@@ -405,10 +406,10 @@ def test_token_major_layout_keeps_strides():
     check_all((o.detach(), rem.detach(), dq, dk, dv), oracle_varlen(q, k, v, do, lengths))
 
 
-@pytest.mark.parametrize("d", [16, 32, 50, 96])
+@pytest.mark.parametrize("d", [16, 32, 50, 96, 160, 200])
 def test_other_head_dims_run_zero_padded(d):
     """Upstream's fixed-length test grid (tests/test_attn.py:39: 64, 32, 16, 50).  32 has kernels of its
-    own; 16 is padded to 32, 50 to 64, 96 to 128."""
+    own; 16 is padded to 32, 50 to 64, 96 to 128, 160 and 200 to 256."""
     from stickbreaking_attention import sb_attn
     q, k, v, do = orc.make_inputs((1, 2, 200, d), d, dist="upstream")
     qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))

@@ -24,7 +24,7 @@ def _need_gpu():
 
 
 @pytest.mark.parametrize("ac", [False, True])
-@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
 @pytest.mark.parametrize("product_space", [False, True])
 def test_varlen_attention_weights(ac, d, product_space, monkeypatch):
     from stickbreaking_attention import _ops
