@@ -4,7 +4,7 @@ A "step" is one forward + backward of sb_attn_varlen over the headline workload 
 32 heads, head_dim 128, 16384 packed tokens in 8 documents, bf16, inputs resident in HBM).
 Prints ONE JSON line: whole-job fwd+bwd TFLOP/s on the causal FLOP count, the roofline of the
 dominant kernel (duration measured with HIP events on the launch stream, inside libsba.so),
-the other BASELINE workloads (c2, c4, c5) measured the same way in the same run, and the CPU
+the other BASELINE workloads (c2, c4, c5) and a head_dim 256 run (d256) measured the same way in the same run, and the CPU
 oracle timed on this host: the dense sb_ref restatement on config c1 and the running-sum
 form on a bounded sample of the headline workload.
 """
@@ -44,11 +44,13 @@ def workload(name):
     if name == "c2":   # fixed-length sb_attn: batch 4 x 16 heads x 2048 tokens x d=64, every (batch, head) one document
         return [2048] * 4, dict(H=16, d=64, scale=1.0, zero_start=False, backward=True, fixed=True, bound="mfma")
     with open(os.path.join(ROOT, "tests", "golden", "doc_lengths.json")) as f:
-        lengths = json.load(f)[name]
+        lengths = json.load(f)["c3" if name == "d256" else name]
     cfg = {"c3": dict(H=32, d=128, scale=1.0, zero_start=False, backward=True, bound="mfma"),
            # many short documents: ~9 GFLOP of forward work against 256 MiB of mandatory traffic -> HBM bound
            "c4": dict(H=32, d=64, scale=1.0, zero_start=True, backward=True, bound="hbm"),
-           "c5": dict(H=32, d=128, scale=0.5, zero_start=False, backward=False, bound="mfma")}[name]
+           "c5": dict(H=32, d=128, scale=0.5, zero_start=False, backward=False, bound="mfma"),
+           # not a BASELINE workload: c3's documents with half the heads at twice the head_dim (the same FLOP count)
+           "d256": dict(H=16, d=256, scale=1.0, zero_start=False, backward=True, bound="mfma")}[name]
     return lengths, cfg
 
 
@@ -255,13 +257,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--ramp-ms", type=float, default=400.0,
                     help="untimed repetitions of the step before the warm-up, until the device clock has settled")
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "d256"])
     ap.add_argument("--lengths", default=None,
                     help="comma-separated document lengths replacing the workload's own (shape sweeps; "
                          "heads, head_dim and scaling stay those of --workload)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true",
-                    help="skip the other BASELINE workloads (c2, c4, c5) that a default run measures beside c3")
+                    help="skip the other workloads (c2, c4, c5, d256) that a default run measures beside c3")
     ap.add_argument("--log-space", action="store_true", help="log2-sum carry instead of product carry")
     ap.add_argument("--epilogue", default="none", choices=["none", "torch", "fused"],
                     help="also form o + rem[..., None] * v, what callers do next (and differentiate through it): "
@@ -321,7 +323,7 @@ def main():
         # the other BASELINE workloads, same method, fewer steps: measured in the same run so that
         # whoever runs this script sees them (they are not the headline metric)
         sec = {}
-        for w in ("c2", "c4", "c5"):
+        for w in ("c2", "c4", "c5", "d256"):
             s = measure(w, max(5, args.steps // 2), 3, args, torch, lib)
             fl = (14.0 if s["backward"] else 4.0) * s["d"] * s["pairs"]
             by = (11.0 if s["backward"] else 4.0) * s["tensor_bytes"]

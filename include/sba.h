@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define SBA_VERSION 212
+#define SBA_VERSION 213
 
 /* error codes (negative returns) */
 #define SBA_E_NULL      (-1)  /* a required pointer is NULL                         */

@@ -989,25 +989,25 @@ __global__ void __launch_bounds__(NT2, 1) bwd_dkdv_kernel(const KArgs a) {
 // and dv.  One barrier (after the Q / dO rows have landed), two workgroups per CU.
 //
 // STREAM: the same four independent waves on EVERY key tile, whatever number of queries follows
-// it: the Q / dO rows then come one query block at a time through two LDS buffers, with one
-// barrier per block.  This is the whole dk/dv pass of head_dim 256, where a wave's K and V
-// fragments (128 registers) and its dk and dv accumulators (256) need the register file of a
-// SIMD to themselves: one workgroup per CU, one wave per SIMD, nothing to split into roles.
+// it: the Q / dO rows then come 64 at a time through two LDS buffers, with one barrier per 64
+// rows (one per 32 rows costs a quarter more time: the waves wait for one another at each).
+// This is the whole dk/dv pass of head_dim 256, where a wave's K and V fragments (128 registers)
+// and the accumulators of ONE of dk and dv (128) with the chains' own temporaries need the
+// register file of a SIMD to themselves: one workgroup per CU, one wave per SIMD, nothing to
+// split into roles, and two passes over the queries, dv first and dk second (both outputs'
+// accumulators at once leave the chains no accumulation registers: 150 to 210 spilled values,
+// whether or not the V fragments wait in LDS instead).
 // -------------------------------------------------------------------------------------------
 template <int D> struct StreamKernel { static constexpr bool value = D > 128; };
 
 template <int D, bool AC, bool PROD, bool STREAM>
 __global__ void __launch_bounds__(NT, D > 128 ? 1 : 2) bwd_dkdv_tail_kernel(const KArgs a) {
   constexpr int KS = D / 16, DB = D / 32;
-  constexpr int SEG = 32;                             // STREAM: query rows per buffer
+  constexpr int SEG = 64;                             // STREAM: query rows per buffer
   constexpr int QROWS = STREAM ? 2 * SEG : TAIL_TILES * BKV;   // rows the buffers hold (not STREAM: every query that can follow the tile's first key)
   __shared__ __attribute__((aligned(16))) unsigned short Qs[QROWS * D];   // Q rows from the tile's first key on (swizzled like every tile)
   __shared__ __attribute__((aligned(16))) unsigned short Gs[QROWS * D];   // dO rows
   __shared__ __attribute__((aligned(16))) unsigned short St[NT / 64][2][32 * 32];   // per wave: p and dz of one block, [query][key]
-  // head_dim 256: a wave's dk and dv accumulators fill the 256 accumulation registers and its K fragments 64
-  // of the others; its V fragments wait in LDS instead, in fragment order (wave-private: no barrier involved)
-  constexpr bool V_IN_LDS = D > 128;
-  __shared__ __attribute__((aligned(16))) unsigned short Vf[V_IN_LDS ? NT / 64 : 1][V_IN_LDS ? KS * 64 * 8 : 8];
 
   const int* sched = a.sched;
   const int4 hdr = *reinterpret_cast<const int4*>(sched);   // status, query tiles, key tiles, table entries needed
@@ -1049,22 +1049,11 @@ __global__ void __launch_bounds__(NT, D > 128 ? 1 : 2) bwd_dkdv_tail_kernel(cons
   const int kblk = (w + blockIdx.x) & (BKV / 32 - 1);
   const int k0 = q_first + 32 * kblk;                // this wave's keys
   const bool active = k0 < L;
-  el8 kf[KS], vf[V_IN_LDS ? 1 : KS];                 // MFMA row n holds key k0 + kperm(n)
+  el8 kf[KS], vf[KS];                                // MFMA row n holds key k0 + kperm(n)
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
     kf[ks] = load_frag(krows, k0 + kperm(n), 32 * ks + 16 * h);
-    if constexpr (!V_IN_LDS) vf[ks] = load_frag(vrows, k0 + kperm(n), 32 * ks + 16 * h);
-  }
-  unsigned short* const Vw = Vf[V_IN_LDS ? w : 0] + 8 * lane;   // this lane's fragment ks at Vw + 512 * ks
-  if constexpr (V_IN_LDS) {
-#pragma unroll
-    for (int c0 = 0; c0 < KS; c0 += 4) {
-      el8 part[4];
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) part[ks] = load_frag(vrows, k0 + kperm(n), 32 * (c0 + ks) + 16 * h);
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) *reinterpret_cast<el8*>(Vw + 512 * (c0 + ks)) = part[ks];
-    }
+    vf[ks] = load_frag(vrows, k0 + kperm(n), 32 * ks + 16 * h);
   }
   // A block that starts past the end of the document is never visible; its table reads are
   // redirected into the document's area and never used.
@@ -1143,10 +1132,7 @@ __global__ void __launch_bounds__(NT, D > 128 ? 1 : 2) bwd_dkdv_tail_kernel(cons
 #pragma unroll
         for (int ks = 0; ks < CH; ++ks) {
           x = mfma32(kf[c0 + ks], qfr[ks], x);
-          if constexpr (DK) {
-            if constexpr (V_IN_LDS) da = mfma32(lds_row8(Vw + 512 * (c0 + ks)), gfr[ks], da);
-            else da = mfma32(vf[c0 + ks], gfr[ks], da);
-          }
+          if constexpr (DK) da = mfma32(vf[c0 + ks], gfr[ks], da);
         }
         if constexpr (D > 128) __builtin_amdgcn_sched_barrier(0);
       }
@@ -1215,24 +1201,29 @@ __global__ void __launch_bounds__(NT, D > 128 ? 1 : 2) bwd_dkdv_tail_kernel(cons
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     store_block32<D>(Pt, acc_k, a.inv_temp, dkb, a.dk.st, k0, L, lane);
   } else {
-    // Two passes over the queries, dv first and dk second: one output's accumulators (128 registers at
-    // head_dim 256) beside the chains' own, instead of both.  The scores are formed in each pass.
-    // Query block s sits in buffer s & 1.  At its top every wave is done with block s - 1, whose buffer
-    // takes the rows of block s + 1 while this one is worked on.
-    static_assert(!STREAM || (QROWS == 64 && NT / 64 == 4), "a quarter of the two buffers per wave for its output");
+    // Two passes over the queries, dv first and dk second; the scores are formed in each.
+    // Segment s (SEG query rows) sits in buffer s & 1.  At its top every wave is done with segment s - 1,
+    // whose buffer takes the rows of segment s + 1 while this one is worked on.
+    static_assert(!STREAM || (QROWS >= 64 && NT / 64 == 4), "a quarter of the first 64 rows of the two buffers per wave for its output");
     unsigned short* const scratch = (w & 2 ? Gs : Qs) + (w & 1) * 32 * D;
+    constexpr int BPS = SEG / 32;                     // query blocks per segment
+    const int nseg = (nblk + BPS - 1) / BPS;
     auto pass = [&](auto what_tag) {
       f32x16 acc[DB];
       clear(acc);
 #pragma unroll 1
-      for (int qblk = 0; qblk < nblk; ++qblk) {
+      for (int sgm = 0; sgm < nseg; ++sgm) {
         wait_loads<0>();
         lds_barrier();
-        if (qblk + 1 < nblk) {
-          qcopy.issue(qrows, q_first + (qblk + 1) * SEG, Qs + ((qblk + 1) & 1) * SEG * D);
-          gcopy.issue(grows, q_first + (qblk + 1) * SEG, Gs + ((qblk + 1) & 1) * SEG * D);
+        if (sgm + 1 < nseg) {
+          qcopy.issue(qrows, q_first + (sgm + 1) * SEG, Qs + ((sgm + 1) & 1) * SEG * D);
+          gcopy.issue(grows, q_first + (sgm + 1) * SEG, Gs + ((sgm + 1) & 1) * SEG * D);
         }
-        if (active && qblk >= kblk) block(what_tag, acc, acc, qblk, (qblk & 1) * SEG);
+#pragma unroll
+        for (int b = 0; b < BPS; ++b) {
+          const int qblk = BPS * sgm + b;
+          if (active && qblk >= kblk && qblk < nblk) block(what_tag, acc, acc, qblk, (sgm & 1) * SEG + 32 * b);
+        }
       }
       lds_barrier();            // every wave is done with the buffers: they become the output staging
       if (active) {

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for s in syms:
         assert hasattr(lib, s), f"{s} declared in include/sba.h but not exported"
     assert sorted(nat.EXPORTS) == syms
-    assert lib.sba_version() == 212
+    assert lib.sba_version() == 213
 
 
 def problem(**kw):
