@@ -32,10 +32,10 @@ PEAK_HBM_GBS = 8000.0       # MI355X published HBM3E bandwidth
 #   mfma_busy, valu_busy, coexec: fractions of the launch's SIMD-cycles in which the matrix pipe is busy
 #     (SQ_VALU_MFMA_BUSY_CYCLES), a vector instruction is active (4 x SQ_ACTIVE_INST_VALU) and both at once
 #     (SQ_VALU_MFMA_COEXEC_CYCLES), over 1024 SIMDs x GRBM_GUI_ACTIVE / 8: profiles/c3_sq_counters_pmc.txt
-MEASURED = {"sba_version": 211,
-            "c3": {"fwd_kernel": {"traffic": 1.090e9, "mfma_busy": 0.468, "valu_busy": 0.560, "coexec": 0.196},
-                   "bwd_dq_kernel": {"traffic": 1.109e9, "mfma_busy": 0.429, "valu_busy": 0.580, "coexec": 0.167},
-                   "bwd_dkdv_kernel": {"traffic": 1.225e9, "mfma_busy": 0.421, "valu_busy": 0.502, "coexec": 0.181}}}
+MEASURED = {"sba_version": 213,
+            "c3": {"fwd_kernel": {"traffic": 1.097e9, "mfma_busy": 0.462, "valu_busy": 0.554, "coexec": 0.193},
+                   "bwd_dq_kernel": {"traffic": 1.108e9, "mfma_busy": 0.428, "valu_busy": 0.578, "coexec": 0.166},
+                   "bwd_dkdv_kernel": {"traffic": 1.228e9, "mfma_busy": 0.421, "valu_busy": 0.503, "coexec": 0.181}}}
 
 KERNELS = ["fwd_kernel", "bwd_dq_kernel", "bwd_dkdv_kernel"]
 
