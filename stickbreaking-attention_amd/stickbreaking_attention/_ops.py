@@ -49,6 +49,13 @@ SYNC_FREE = os.environ.get("SBA_SYNC_FREE", "0") == "1"
 # rebuilt table is one scratch buffer shared by all layers.
 RECOMPUTE_TABLE = os.environ.get("SBA_RECOMPUTE_TABLE", "0") == "1"
 
+# With SBA_F32_AS_F16=1 float32 inputs run on the float16 kernels instead of being rounded to bfloat16: operands of 11
+# significant bits, what upstream's tl.dot gives float32 inputs with TF32 allowed (utils.py:8, sb_varlen_fwd.py:42),
+# against bfloat16's 8.  float16 has a narrow exponent: q, k, v must stay within +-65504 (beyond that the outputs are
+# NaN), which is why this is a switch and not the default; the incoming gradient, whose scale is arbitrary, is brought
+# to a maximum between 4 and 8 by a power of two before it is rounded and the gradients are scaled back (exact).
+F32_AS_F16 = os.environ.get("SBA_F32_AS_F16", "0") == "1"
+
 SUPPORTED_HEAD_DIMS = (32, 64, 128, 256)
 
 # Tile sizes the library's workspace formulas are built on (query tile, dk/dv key tile, table block).
@@ -205,8 +212,10 @@ def _warn_reduced_precision(dtype) -> None:
 
 def compute_dtype(dtype: torch.dtype) -> torch.dtype:
     """The element type the kernels run in for inputs of `dtype`: bfloat16 and float16 natively (MFMA
-    of that type, fp32 accumulation), everything else in bfloat16."""
-    return dtype if dtype in (torch.bfloat16, torch.float16) else torch.bfloat16
+    of that type, fp32 accumulation), everything else in bfloat16 (float32 in float16 with F32_AS_F16)."""
+    if dtype in (torch.bfloat16, torch.float16):
+        return dtype
+    return torch.float16 if (dtype == torch.float32 and F32_AS_F16) else torch.bfloat16
 
 
 def _prep(t: torch.Tensor, dpad: int, cdt: torch.dtype, incoming_grad: bool = False) -> torch.Tensor:
@@ -214,7 +223,7 @@ def _prep(t: torch.Tensor, dpad: int, cdt: torch.dtype, incoming_grad: bool = Fa
     (traceable).  The strides of an incoming gradient are not known while a backward is being
     traced, so there it is simply made contiguous."""
     if t.dtype != cdt:
-        if not torch.compiler.is_compiling() and t.dtype not in (torch.bfloat16, torch.float16):
+        if not torch.compiler.is_compiling() and t.dtype not in (torch.bfloat16, torch.float16) and cdt == torch.bfloat16:
             _warn_reduced_precision(t.dtype)
         t = t.to(cdt)
     d = t.shape[-1]
@@ -541,6 +550,19 @@ def run_backward(q, k, v, do, drem, fixed: bool, state, inv_temp: float, attend_
     dpad = _padded_dim(d)
     cdt = compute_dtype(q.dtype)
     qp, kp, vp = (_prep(t, dpad, cdt) for t in (q, k, v))
+    unscale = None
+    if cdt == torch.float16 and q.dtype == torch.float32:
+        # float32 caller on the float16 kernels: a power of two brings the largest incoming gradient into [4, 8)
+        # (the backward is linear in (do, drem); no value is read back to the host)
+        amax = do.detach().abs().amax().float()
+        if drem is not None:
+            amax = torch.maximum(amax, drem.detach().abs().amax().float())
+        expo = torch.floor(torch.log2(amax.clamp(min=2.0 ** -100, max=2.0 ** 100)))
+        scale = torch.exp2(2.0 - expo)
+        unscale = torch.exp2(expo - 2.0)
+        do = do.float() * scale
+        if drem is not None:
+            drem = drem.float() * scale
     dop = _prep(do, dpad, cdt, incoming_grad=True)
     if drem is None:
         dremp = torch.empty(0, dtype=cdt, device=q.device)
@@ -559,6 +581,8 @@ def run_backward(q, k, v, do, drem, fixed: bool, state, inv_temp: float, attend_
     else:
         _compileable_backward(dop, dremp, qp, kp, vp, cu, max_len, float(inv_temp), bool(attend_current),
                               product, bool(fused), table, sched, gtab, dq, dk, dv)
+    if unscale is not None:
+        dq, dk, dv = (t[..., :d].float() * unscale for t in (dq, dk, dv))
     if dpad != d or q.dtype != cdt or k.dtype != cdt or v.dtype != cdt or dkdv_dtype not in (None, cdt):
         dq = dq[..., :d].to(q.dtype)
         dk = dk[..., :d].to(k.dtype if dkdv_dtype is None else dkdv_dtype)

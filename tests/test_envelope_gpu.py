@@ -81,6 +81,48 @@ def test_fp32_inputs_are_rounded_to_bf16_and_say_so():
         assert_close(name + " (fp32 inputs)", gt, r)
 
 
+@pytest.mark.parametrize("gscale", [1.0, 1e-6, 3e4])
+def test_float32_inputs_on_the_float16_kernels(gscale, monkeypatch):
+    """SBA_F32_AS_F16: float32 callers get operands of 11 significant bits (what TF32 gives upstream's float32
+    dots, utils.py:8) instead of bfloat16's 8.  The incoming gradient may have any scale -- 1e-6 would be a
+    float16 subnormal, 3e4 * sqrt(d) would overflow dz -- so it is normalised by a power of two and the gradients
+    scaled back: the error relative to the gradient's scale must not depend on it, and must be several times
+    below what the bfloat16 route gives on the same values.  No precision warning; float32 outputs."""
+    from stickbreaking_attention import _ops, sb_attn_varlen
+    lengths = [257, 640, 95]
+    T = sum(lengths)
+    g = torch.Generator().manual_seed(4321)
+    q, k, v, do = (torch.randn((3, T, 64), generator=g) for _ in range(4))
+    do = do * gscale
+    drem = torch.randn((3, T), generator=g) * gscale
+    ref = orc.sb_varlen_grads(q, k, v, lengths, do, drem)
+    cu = cu_from_lengths(lengths, device=DEV)
+
+    def run():
+        qg, kg, vg = (t.to(DEV).requires_grad_() for t in (q, k, v))
+        o, rem = sb_attn_varlen(qg, kg, vg, cu, max(lengths), zero_start=False)
+        grads = torch.autograd.grad((o, rem), (qg, kg, vg), (do.to(DEV), drem.to(DEV)))
+        torch.cuda.synchronize()
+        return (o.detach(), rem.detach()) + grads
+
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        coarse = run()                                  # the default: rounded to bfloat16
+    monkeypatch.setattr(_ops, "F32_AS_F16", True)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        fine = run()
+    for name, gt, gc, r in zip(("o", "rem", "dq", "dk", "dv"), fine, coarse, ref):
+        assert gt.dtype == torch.float32
+        unit = 1.0 if name in ("o", "rem") else gscale
+        diff = (gt.cpu() - r).abs()
+        worse = (gc.cpu() - r).abs().max().item()
+        print(f"  {name} (float32 on float16 kernels, gradient scale {gscale:g}): max_abs={diff.max().item():.3e}, "
+              f"rounded to bfloat16: {worse:.3e}")
+        assert (diff <= 4e-3 * unit + r.abs() * 2.0 ** -11).all(), f"{name}: {diff.max().item():.3e}"
+        assert diff.max().item() * 3 < worse, f"{name}: not clearly finer than the bfloat16 route"
+
+
 @pytest.mark.parametrize("d", [32, 64, 128, 256])
 def test_float16_runs_on_the_float16_kernels(d):
     """float16 q, k, v, grad_o are multiplied as float16 (11 significant bits instead of bfloat16's 8;
